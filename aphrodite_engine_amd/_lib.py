@@ -162,6 +162,22 @@ SIGNATURES = {
                                              F, F, F, P, I, I, I, P, Z, P]),
 }
 
+# libaphrodite_mi355x_mixers.so (include/aphrodite_mi355x_mixers.h): the sequence-mixer kernels, a library of its own so that
+# a model built from them alone needs nothing else compiled
+MIXERS_LIB_PATH = os.environ.get(
+    "APHRODITE_MI355X_MIXERS_LIB", os.path.join(_HERE, "lib", "libaphrodite_mi355x_mixers.so"))
+MIXERS_SIGNATURES = {
+    "aphro_mixers_last_error": (ctypes.c_char_p, []),
+    "aphro_embed_scale_f32": (I, [P, P, P, L, I, L, F, I, P]),
+    "aphro_residual_layer_norm": (I, [P, P, L, P, P, P, P, P, P, P, L, I, F, I, P]),
+    "aphro_act_and_mul": (I, [P, P, L, L, I, I, I, P]),
+    "aphro_gated_group_rms_norm": (I, [P, L, P, P, P, L, L, I, I, F, F, I, P]),
+    "aphro_paged_kv_write": (I, [P, P, P, L, P, L, P, L, I, I, I, L, I, P]),
+    "aphro_distance_bias_attention": (I, [P, L, P, L, P, L, P, P, P, I, L, I, P, P, P, L, I, I, I, I, I, F, P, I, F, I, F,
+                                          I, P]),
+    "aphro_outer_memory_scan": (I, [P, P, L, P, L, P, L, P, P, L, P, P, P, P, I, P, P, P, I, L, I, I, I, I, P, F, F, I, P]),
+}
+
 OK = 0
 F16, BF16, F32 = 0, 1, 2
 KV_AUTO, KV_FP8_E4M3, KV_FP8_E5M2 = 0, 1, 2
@@ -189,6 +205,46 @@ def lib():
         fn.argtypes = args
     _lib = l
     return l
+
+
+_mixers = None
+
+
+def build_mixers() -> None:
+    """Compile libaphrodite_mi355x_mixers.so in the tree (hipcc, gfx950; a few seconds per file)."""
+    import subprocess
+    src = os.path.join(_HERE, "csrc", "mixers")
+    r = subprocess.run(["make", "-C", src, "-j", "4"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise ImportError("building libaphrodite_mi355x_mixers.so failed:\n" + r.stdout[-4000:])
+
+
+def mixers_lib():
+    """Load the mixer kernels (once).  Built on first use when the tree holds no library yet; like ``lib()`` there is no
+    CPU fallback behind it."""
+    global _mixers
+    if _mixers is not None:
+        return _mixers
+    if not os.path.exists(MIXERS_LIB_PATH):
+        if "APHRODITE_MI355X_MIXERS_LIB" in os.environ:
+            raise ImportError(f"{MIXERS_LIB_PATH} not found")
+        build_mixers()
+    l = ctypes.CDLL(MIXERS_LIB_PATH)
+    for name, (res, args) in MIXERS_SIGNATURES.items():
+        try:
+            fn = getattr(l, name)
+        except AttributeError as e:
+            raise ImportError(f"{MIXERS_LIB_PATH} does not export {name}") from e
+        fn.restype = res
+        fn.argtypes = args
+    _mixers = l
+    return l
+
+
+def check_mixers(rc, what=""):
+    if rc != OK:
+        msg = mixers_lib().aphro_mixers_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what}: {msg} (code {rc})" if what else f"{msg} (code {rc})")
 
 
 def check(rc, what=""):

@@ -473,10 +473,19 @@ def read_kv_cache_scales(path: str, tp_rank: int, tp_size: int, num_hidden_layer
 def load_model(model_dir: str, dtype: torch.dtype = torch.float16, kv_cache_dtype: str = "auto",
                device: Union[str, torch.device] = "cuda", quantization: Optional[str] = None,
                quantization_param_path: Optional[str] = None, process_weights: bool = True):
-    """config.json + quantisation config + *.safetensors -> a ready LlamaForCausalLM on ``device``
-    (the role of DefaultModelLoader.load_model, model_loader/loader.py:370-420)."""
-    from .model import LlamaForCausalLM, _rope_cache
+    """config.json + *.safetensors -> a ready model on ``device``: the class is chosen by the architecture that config.json
+    names (registry.py; the role of DefaultModelLoader.load_model, model_loader/loader.py:370-420)."""
+    from .registry import resolve
     hf = read_hf_config(model_dir)
+    return resolve(hf)(model_dir, hf, dtype=dtype, kv_cache_dtype=kv_cache_dtype, device=device, quantization=quantization,
+                       quantization_param_path=quantization_param_path, process_weights=process_weights)
+
+
+def load_llama_model(model_dir: str, hf: Dict[str, Any], dtype: torch.dtype = torch.float16, kv_cache_dtype: str = "auto",
+                     device: Union[str, torch.device] = "cuda", quantization: Optional[str] = None,
+                     quantization_param_path: Optional[str] = None, process_weights: bool = True):
+    """The Llama family: quantisation config + weights -> LlamaForCausalLM."""
+    from .model import LlamaForCausalLM, _rope_cache
     cfg = llama_config_from_hf(hf)
     qc = resolve_quant_config(model_dir, hf, quantization, dtype)
     model = LlamaForCausalLM(cfg, qc, dtype, kv_cache_dtype)

@@ -1,0 +1,222 @@
+"""Torch-tensor front of libaphrodite_mi355x_mixers.so (include/aphrodite_mi355x_mixers.h), in the manner of
+``_custom_ops``: every wrapper checks on the host what the kernel and its grid assume (shapes, strides, dtypes, devices)
+before it launches, issues on the current stream, allocates only its result, and raises on CPU tensors -- there is no
+fallback."""
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import check_mixers as check
+
+_DT = {torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+ACT_SILU, ACT_GELU_TANH = 0, 1
+MEMORY_DECAY, MEMORY_MLSTM = 0, 1
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise RuntimeError(f"mixer ops serve bfloat16 and float32 activations, not {t.dtype}")
+    return _DT[t.dtype]
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _cuda(*ts) -> None:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("mixer ops run on the GPU only (no CPU fallback)")
+        dev = dev or t.device
+        _need(t.device == dev, "mixer ops: tensors on different devices")
+
+
+def _rows(t: torch.Tensor, cols: int, what: str) -> int:
+    """Row stride (elements) of a [T, cols] view whose rows are dense."""
+    _need(t.dim() == 2 and t.shape[1] == cols and (t.stride(1) == 1 or cols == 1), f"{what}: expected dense rows of {cols}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), cols)
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor, n: int, what: str) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n, f"{what}: int32 [{n}] expected")
+
+
+def embed_scale(table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 residual rows ``table[ids] * scale``."""
+    _cuda(table, ids)
+    _need(table.dim() == 2 and table.is_contiguous() and ids.dtype == torch.int64 and ids.dim() == 1 and ids.is_contiguous(),
+          "embed_scale: table [vocab, width] contiguous, ids int64 [T]")
+    out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+    check(_lib.mixers_lib().aphro_embed_scale_f32(out.data_ptr(), table.data_ptr(), ids.data_ptr(), ids.shape[0],
+                                                  table.shape[1], table.shape[0], float(scale), _dt(table), _stream()),
+          "embed_scale")
+    return out
+
+
+def residual_layer_norm(residual: torch.Tensor, y: Optional[torch.Tensor] = None, post=None,
+                        y_bias: Optional[torch.Tensor] = None, add_vec: Optional[torch.Tensor] = None, pre=None,
+                        eps: float = 1e-5, dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """``residual += layer_norm(y + y_bias; *post)``, ``residual += add_vec``, return ``layer_norm(residual; *pre)``; each
+    step only if its operands are given.  ``post`` / ``pre`` are (weight, bias) pairs of the activation dtype."""
+    T, W = residual.shape
+    _need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual_layer_norm: the residual is fp32, contiguous")
+    some = y if y is not None else (pre[0] if pre is not None else add_vec)
+    _need(some is not None, "residual_layer_norm: nothing to do")
+    adt = dtype or some.dtype
+    vecs = [add_vec] + list(post or ()) + list(pre or ())
+    _cuda(residual, y, y_bias, *vecs)
+    for v in vecs:
+        _need(v is None or (v.dtype == adt and v.numel() == W and v.is_contiguous()), "residual_layer_norm: vectors are [width] of the activation dtype")
+    _need(y_bias is None or (y_bias.dtype == torch.float32 and y_bias.numel() == W and y_bias.is_contiguous()),
+          "residual_layer_norm: y_bias is fp32 [width]")
+    ys = 0
+    if y is not None:
+        _need(post is not None and y.dtype == adt and y.shape[0] == T, "residual_layer_norm: y needs its norm and the batch's rows")
+        ys = _rows(y, W, "residual_layer_norm y")
+    out = torch.empty(T, W, dtype=adt, device=residual.device) if pre is not None else None
+    if _dt_of(adt) is None:
+        raise RuntimeError(f"residual_layer_norm: dtype {adt}")
+    check(_lib.mixers_lib().aphro_residual_layer_norm(
+        residual.data_ptr(), _p(y), ys, _p(y_bias), _p(post[0]) if post else None, _p(post[1]) if post else None,
+        _p(add_vec), _p(pre[0]) if pre else None, _p(pre[1]) if pre else None, _p(out), T, W, float(eps), _DT[adt], _stream()),
+        "residual_layer_norm")
+    return out
+
+
+def _dt_of(dtype):
+    return _DT.get(dtype)
+
+
+def act_and_mul(x: torch.Tensor, act: int) -> torch.Tensor:
+    """[T, 2 d] -> [T, d]: act(x[:, :d]) * x[:, d:]."""
+    _cuda(x)
+    _need(x.dim() == 2 and x.shape[1] % 2 == 0, "act_and_mul: [T, 2 d]")
+    d = x.shape[1] // 2
+    out = torch.empty(x.shape[0], d, dtype=x.dtype, device=x.device)
+    check(_lib.mixers_lib().aphro_act_and_mul(out.data_ptr(), x.data_ptr(), _rows(x, 2 * d, "act_and_mul"), x.shape[0], d,
+                                              int(act), _dt(x), _stream()), "act_and_mul")
+    return out
+
+
+def gated_group_rms_norm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                         group: int, eps: float, out_scale: float = 1.0) -> None:
+    """out[:, :N] (a view with dense rows, any row stride) = out_scale * x / rms(x per group) * weight * sigmoid(gate)."""
+    _cuda(out, x, weight, gate)
+    T, N = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "gated_group_rms_norm: x is fp32 contiguous")
+    _need(out.shape == (T, N) and N % group == 0, "gated_group_rms_norm: out [T, N], N a multiple of the group")
+    _need(weight is None or (weight.dtype == out.dtype and weight.numel() == N and weight.is_contiguous()), "gated_group_rms_norm: weight [N]")
+    gs = 0
+    if gate is not None:
+        _need(gate.dtype == out.dtype and gate.shape == (T, N), "gated_group_rms_norm: gate [T, N] of the output dtype")
+        gs = _rows(gate, N, "gated_group_rms_norm gate")
+    check(_lib.mixers_lib().aphro_gated_group_rms_norm(out.data_ptr(), _rows(out, N, "gated_group_rms_norm out"), x.data_ptr(),
+                                                       _p(weight), _p(gate), gs, T, N, int(group), float(eps),
+                                                       float(out_scale), _dt(out), _stream()), "gated_group_rms_norm")
+
+
+def paged_kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                   slot_mapping: torch.Tensor) -> None:
+    """k_cache [blocks, block, G, d], v_cache [blocks, block, G, e]; k [T, G d], v [T, G e] (dense rows); slots int64 [T]."""
+    _cuda(k_cache, v_cache, k, v, slot_mapping)
+    nb, bs, G, d = k_cache.shape
+    e = v_cache.shape[3]
+    _need(v_cache.shape[:3] == (nb, bs, G) and k_cache.is_contiguous() and v_cache.is_contiguous(), "paged_kv_write: cache shapes")
+    _need(k.dtype == k_cache.dtype == v.dtype == v_cache.dtype, "paged_kv_write: one dtype")
+    T = k.shape[0]
+    _need(v.shape[0] == T and slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous(),
+          "paged_kv_write: slots int64 [T]")
+    check(_lib.mixers_lib().aphro_paged_kv_write(k_cache.data_ptr(), v_cache.data_ptr(), k.data_ptr(), _rows(k, G * d, "k"),
+                                                 v.data_ptr(), _rows(v, G * e, "v"), slot_mapping.data_ptr(), T, G, d, e,
+                                                 nb * bs, _dt(k), _stream()), "paged_kv_write")
+
+
+def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor,
+                            v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
+                            seq_of_token: torch.Tensor, heads: int, scale: float, bias_lut: Optional[torch.Tensor],
+                            temp_coef: float = 0.0, temp_every: int = 1, out_scale: float = 1.0) -> None:
+    """Causal attention of a batch of segments over the paged cache, written into ``out`` [T, heads * e] (dense rows, any
+    row stride).  q [T, heads * d]; gate [T, heads] raw (sigmoid inside) or None; bias_lut fp32 [heads, L] indexed by
+    min(distance, L - 1) or None."""
+    _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, ctx_len, seq_of_token, bias_lut)
+    nb, bs, G, d = k_cache.shape
+    e = v_cache.shape[3]
+    T = q.shape[0]
+    S = q_start.numel()
+    _need(v_cache.shape[:3] == (nb, bs, G) and k_cache.is_contiguous() and v_cache.is_contiguous(), "distance_bias_attention: cache shapes")
+    _need(q.dtype == out.dtype == k_cache.dtype == v_cache.dtype, "distance_bias_attention: one dtype")
+    _need(heads % G == 0 and out.shape == (T, heads * e), "distance_bias_attention: out [T, heads * vdim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.is_contiguous(),
+          "distance_bias_attention: block_tables int32 [S, max_blocks]")
+    _i32(q_start, S, "q_start")
+    _i32(ctx_len, S, "ctx_len")
+    _i32(seq_of_token, T, "seq_of_token")
+    gs = 0
+    if gate is not None:
+        _need(gate.dtype == q.dtype and gate.shape[0] == T, "distance_bias_attention: gate [T, heads]")
+        gs = _rows(gate, heads, "gate")
+    L = 0
+    if bias_lut is not None:
+        _need(bias_lut.dtype == torch.float32 and bias_lut.dim() == 2 and bias_lut.shape[0] == heads and bias_lut.is_contiguous(),
+              "distance_bias_attention: bias_lut fp32 [heads, L]")
+        L = bias_lut.shape[1]
+    check(_lib.mixers_lib().aphro_distance_bias_attention(
+        out.data_ptr(), _rows(out, heads * e, "out"), q.data_ptr(), _rows(q, heads * d, "q"), _p(gate), gs, k_cache.data_ptr(),
+        v_cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(),
+        seq_of_token.data_ptr(), T, S, heads, G, d, e, float(scale), _p(bias_lut), L, float(temp_coef), int(temp_every),
+        float(out_scale), _dt(q), _stream()), "distance_bias_attention")
+
+
+def memory_state_shapes(slots: int, heads: int, dim: int, vdim: int, mode: int):
+    """Shapes of the fp32 state tensors of ``outer_memory_scan`` for a pool of ``slots`` requests."""
+    tiles = (vdim + 63) // 64
+    s = (slots, heads, dim, vdim)
+    return (s, ) if mode == MEMORY_DECAY else (s, (slots, heads, tiles, dim), (slots, heads, tiles))
+
+
+def outer_memory_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state, slot_of_seq: torch.Tensor,
+                      q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, heads: int, mode: int,
+                      decay: Optional[torch.Tensor] = None, gate_i: Optional[torch.Tensor] = None,
+                      gate_f: Optional[torch.Tensor] = None, q_scale: float = 1.0, gate_cap: float = 1.0) -> torch.Tensor:
+    """Scan every segment through its slot's state (updated in place); returns o fp32 [T, heads * vdim].  ``state`` is
+    the tuple of tensors shaped by ``memory_state_shapes``.  q, k [T, heads * d], v [T, heads * e]; gates [T, heads] raw."""
+    _cuda(q, k, v, slot_of_seq, q_start, q_len, ctx_len, decay, gate_i, gate_f, *state)
+    T = q.shape[0]
+    S = q_start.numel()
+    slots, H, d, e = state[0].shape
+    _need(H == heads and k.shape[0] == T and v.shape[0] == T and q.dtype == k.dtype == v.dtype, "outer_memory_scan: q, k, v rows / dtype")
+    for st, shp in zip(state, memory_state_shapes(slots, heads, d, e, mode)):
+        _need(st.dtype == torch.float32 and st.is_contiguous() and tuple(st.shape) == shp, "outer_memory_scan: state tensors")
+    _need(len(state) == (1 if mode == MEMORY_DECAY else 3), "outer_memory_scan: state tuple")
+    for t, nm in ((slot_of_seq, "slot_of_seq"), (q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    gs = 0
+    if mode == MEMORY_DECAY:
+        _need(decay is not None and decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous(),
+              "outer_memory_scan: decay fp32 [heads]")
+    else:
+        _need(gate_i is not None and gate_f is not None and gate_i.dtype == q.dtype == gate_f.dtype
+              and gate_i.shape[0] == T and gate_f.shape[0] == T, "outer_memory_scan: gates [T, heads]")
+        gs = _rows(gate_i, heads, "gate_i")
+        _need(_rows(gate_f, heads, "gate_f") == gs, "outer_memory_scan: the two gates share a row stride")
+    out = torch.empty(T, heads * e, dtype=torch.float32, device=q.device)
+    check(_lib.mixers_lib().aphro_outer_memory_scan(
+        out.data_ptr(), q.data_ptr(), _rows(q, heads * d, "q"), k.data_ptr(), _rows(k, heads * d, "k"), v.data_ptr(),
+        _rows(v, heads * e, "v"), _p(gate_i), _p(gate_f), gs, state[0].data_ptr(),
+        state[1].data_ptr() if len(state) > 1 else None, state[2].data_ptr() if len(state) > 2 else None,
+        slot_of_seq.data_ptr(), slots, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), S, T, heads, d, e, int(mode),
+        _p(decay), float(q_scale), float(gate_cap), _dt(q), _stream()), "outer_memory_scan")
+    return out

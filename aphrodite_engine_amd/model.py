@@ -1059,6 +1059,21 @@ class LlamaForCausalLM(nn.Module):
         ops.fused_add_rms_norm(hidden, residual, self.norm, self.cfg.rms_norm_eps)
         return hidden
 
+    # ---- what the engine (engine.py) asks of a model ------------------------------------------------------------------
+    @property
+    def vocab_size(self) -> int:
+        return self.cfg.vocab_size
+
+    def make_caches(self, num_blocks: int, block_size: int, num_slots: int, device):
+        """Paged KV caches of every layer (no per-request state: ``num_slots`` only bounds the batch)."""
+        return make_kv_caches(self.cfg, num_blocks, block_size, self.dtype, self.kv_cache_dtype, device, fill=False)
+
+    @torch.no_grad()
+    def step(self, batch, caches, rows):
+        """One engine step over a StepBatch (prompt portions first, decoded tokens last): fp32 logits of ``rows``."""
+        hidden = self(batch.input_ids, batch.positions, caches, batch.attention_metadata())
+        return self.compute_logits(hidden.index_select(0, rows)).float()
+
     def compute_logits(self, hidden):
         logits = torch.matmul(hidden, self.lm_head.t())
         if get_tensor_model_parallel_world_size() > 1:
