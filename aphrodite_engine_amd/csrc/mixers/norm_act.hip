@@ -145,7 +145,7 @@ extern "C" int aphro_residual_layer_norm(float* residual, const void* y, int64_t
                                          const void* pre_b, void* out, int64_t num_tokens, int width, float eps, int dtype,
                                          void* stream) {
   if (num_tokens == 0) return APHRO_OK;
-  APHRO_CHECK(residual && num_tokens > 0 && width > 0 && width <= 32768, "residual_layer_norm: bad sizes (width %d)", width);
+  APHRO_CHECK(residual && num_tokens > 0 && width > 0 && width <= 16000, "residual_layer_norm: bad sizes (width %d)", width);
   APHRO_CHECK(!y || (post_w && post_b && y_stride >= width), "residual_layer_norm: y needs post_w, post_b and a row stride >= width");
   APHRO_CHECK(!out || (pre_w && pre_b), "residual_layer_norm: out needs pre_w and pre_b");
   APHRO_CHECK(y || add_vec || out, "residual_layer_norm: nothing to do");

@@ -217,8 +217,9 @@ class LLMEngine:
         for rid, toks, w in entries:
             r = self.requests.get(rid)
             if r is None:
-                r = self.requests[rid] = Request(rid, [], 0)
-                self._admit(r)
+                r = Request(rid, [], 0)
+                self._admit(r)                 # raises before the request is known if no slot is free
+                self.requests[rid] = r
             toks = [int(t) for t in toks]
             if not self._reserve(r, len(toks)):
                 raise NoFreePages(f"request {rid}: no pages left for {len(toks)} more tokens")
