@@ -1,0 +1,196 @@
+"""``bench.py --mixers``: prefill and decode throughput of a Fatudra stack at sizes that resemble a real model's layers
+(random bf16 weights), beside a Llama stack of equal width / heads / feed-forward / layer count on the unquantised op path,
+plus each mixer kernel alone against its roofline and against the like kernel of the Llama path.  Prints ONE JSON line;
+the default workload of bench.py is untouched by it.
+
+Rooflines used: 8 TB/s HBM for the memory-bound kernels (norms, activations, decode attention, the decode step of the
+memories: their state is read and written once), 2.5 PFLOP/s dense bf16 MFMA for prompt attention (4 d flops per visible
+query-key pair and head), and for the prompt scan of the memories the same MFMA figure over 4 d e flops per token and head
+(what a chunked matrix form would need; the scan kernel itself runs on the vector ALUs)."""
+import json
+import math
+import time
+
+import torch
+
+HBM, MFMA = 8.0e12, 2.5e15
+
+SIZES = {
+    "w2048": dict(width=2048, ff=5632, heads=16, kv_heads=4, dim=128, mem_heads=8, mem_dim=64, mem_vdim=128, ml_heads=4,
+                  ml_dim=128, ml_vdim=256),
+    "w4096": dict(width=4096, ff=11008, heads=32, kv_heads=8, dim=128, mem_heads=16, mem_dim=64, mem_vdim=128, ml_heads=8,
+                  ml_dim=128, ml_vdim=256),
+}
+LAYERS, VOCAB, BLOCK = 4, 32000, 16
+
+
+def fatudra_config(s):
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "bias_max": 4096,
+                              "scale": s["dim"] ** -0.5, "q_temp": {"coef": 0.1, "every": 512}},
+                     "right": {"heads": s["mem_heads"], "dim": s["mem_dim"], "vdim": s["mem_vdim"],
+                               "decay": [1.0 - 2.0 ** -(2 + 6 * i / max(1, s["mem_heads"] - 1)) for i in range(s["mem_heads"])]},
+                     "left_scale": 1.0, "right_scale": 1.0},
+           "mlp": {"kind": "dense", "ff": s["ff"]}}
+    ml = {"type": "mlstm", "mixer": {"heads": s["ml_heads"], "dim": s["ml_dim"], "vdim": s["ml_vdim"], "gate_cap": 15.0},
+          "mlp": {"kind": "dense", "ff": s["ff"]}}
+    return {"architecture": "Fatudra", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "layers": [par, ml, par, par][:LAYERS]}
+
+
+def timed(fn, iters=10, warmup=3):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e-3
+
+
+def batches(prompt_len, batch, ctx, device, vocab):
+    from .step_batch import StepBatch
+    g = torch.Generator().manual_seed(0)
+    pages = (prompt_len + BLOCK - 1) // BLOCK
+    pre = StepBatch.build([torch.randint(0, vocab, (prompt_len, ), generator=g).tolist()], [0], [list(range(pages))], [0], BLOCK,
+                          device)
+    per = (ctx + 1 + BLOCK - 1) // BLOCK
+    perm = torch.randperm(batch * per, generator=g).view(batch, per).tolist()
+    dec = StepBatch.build([[int(t)] for t in torch.randint(0, vocab, (batch, ), generator=g)], [ctx] * batch, perm,
+                          list(range(batch)), BLOCK, device)
+    return pre, dec, max(pages, batch * per)
+
+
+def model_throughput(model, prompt_len, batch, ctx, device, vocab):
+    pre, dec, pages = batches(prompt_len, batch, ctx, device, vocab)
+    caches = model.make_caches(pages, BLOCK, batch, device)
+    rows_p = torch.tensor([prompt_len - 1], device=device)
+    rows_d = torch.arange(batch, device=device)
+    tp = timed(lambda: model.step(pre, caches, rows_p), iters=5, warmup=2)
+    td = timed(lambda: model.step(dec, caches, rows_d), iters=20, warmup=3)
+    return {"prefill_tokens": prompt_len, "prefill_ms": round(tp * 1e3, 3), "prefill_tok_s": round(prompt_len / tp),
+            "decode_batch": batch, "decode_ctx": ctx, "decode_ms": round(td * 1e3, 3), "decode_tok_s": round(batch / td)}
+
+
+def kernel_section(s, prompt_len, batch, ctx, device):
+    """Each mixer kernel alone at the stack's shapes, and the like kernel of the Llama path at the same shapes."""
+    from . import _custom_ops as ops
+    from . import mixer_ops as mops
+    from .mixers import DistanceBiasAttention
+    bf = torch.bfloat16
+    H, G, d, W, ff = s["heads"], s["kv_heads"], s["dim"], s["width"], s["ff"]
+    pre, dec, pages = batches(prompt_len, batch, ctx, device, VOCAB)
+    out = {}
+
+    def rec(name, sec, bytes_=None, flops=None, like=None):
+        r = {"us": round(sec * 1e6, 1)}
+        if bytes_ is not None:
+            r["frac_hbm"] = round(bytes_ / sec / HBM, 3)
+        if flops is not None:
+            r["frac_mfma"] = round(flops / sec / MFMA, 4)
+        if like is not None:
+            r["like"] = like
+        out[name] = r
+        return r
+
+    # ---- attention --------------------------------------------------------------------------------------------------
+    att = DistanceBiasAttention(H, G, d, d, d ** -0.5, bias_rows=32, bias_far=4096.0, temp_coef=0.1, temp_every=512).to(device)
+    att.rel.normal_()
+    att.finalize()
+    kc, vc = att.cache_spec().allocate(pages, BLOCK, batch, bf, device)
+    kc.normal_()
+    vc.normal_()
+    for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+        q = torch.randn(T, H * d, device=device, dtype=bf)
+        gate = torch.randn(T, H, device=device, dtype=bf)
+        o = torch.empty(T, H * d, device=device, dtype=bf)
+        sec = timed(lambda: mops.distance_bias_attention(o, q, gate, kc, vc, b.block_tables, b.q_start, b.q_len, b.ctx_len,
+                                                         b.seq_of_token, (min(b.q_lens), max(b.q_lens)), H, att.scale, att.bias_lut, att.temp_coef, att.temp_every))
+        if name == "prefill":
+            flops = 4.0 * d * H * T * (T + 1) / 2
+            k = torch.randn(T, G, d, device=device, dtype=bf)
+            v = torch.randn(T, G, d, device=device, dtype=bf)
+            cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+            lsec = timed(lambda: ops.flash_attn_varlen(q.view(T, H, d), k, v, cu, T, d ** -0.5, causal=True))
+            rec("attention_prefill", sec, flops=flops, like={"kernel": "flash_attn_varlen", "us": round(lsec * 1e6, 1),
+                                                             "frac_mfma": round(flops / lsec / MFMA, 4)})
+        else:
+            nbytes = batch * (ctx + 1) * G * 2 * d * 2
+            lk = torch.randn(pages, G, d // 8, BLOCK, 8, device=device, dtype=bf)
+            lv = torch.randn(pages, G, d, BLOCK, device=device, dtype=bf)
+            lens = torch.full((batch, ), ctx + 1, dtype=torch.int32, device=device)
+            lo = torch.empty(T, H, d, device=device, dtype=bf)
+            lsec = timed(lambda: ops.paged_attention_v1(lo, q.view(T, H, d), lk, lv, G, d ** -0.5, b.block_tables, lens, BLOCK,
+                                                        ctx + 1, None, "auto", 1.0, 1.0))
+            rec("attention_decode", sec, bytes_=nbytes, like={"kernel": "paged_attention_v1", "us": round(lsec * 1e6, 1),
+                                                              "frac_hbm": round(nbytes / lsec / HBM, 3)})
+    # ---- memories ---------------------------------------------------------------------------------------------------
+    for tag, mode, Hm, dm, em in (("decay_memory", mops.MEMORY_DECAY, s["mem_heads"], s["mem_dim"], s["mem_vdim"]),
+                                  ("mlstm_memory", mops.MEMORY_MLSTM, s["ml_heads"], s["ml_dim"], s["ml_vdim"])):
+        state = tuple(torch.zeros(x, device=device) for x in mops.memory_state_shapes(batch, Hm, dm, em, mode))
+        decay = torch.full((Hm, ), 0.99, device=device)
+        for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+            q = torch.randn(T, Hm * dm, device=device, dtype=bf)
+            k = torch.randn(T, Hm * dm, device=device, dtype=bf)
+            v = torch.randn(T, Hm * em, device=device, dtype=bf)
+            gi, gf = torch.randn(T, Hm, device=device, dtype=bf), torch.randn(T, Hm, device=device, dtype=bf) + 3
+            sec = timed(lambda: mops.outer_memory_scan(q, k, v, state, b.state_slots, b.q_start, b.q_len, b.ctx_len, Hm, mode,
+                                                       decay=decay, gate_i=gi, gate_f=gf, q_scale=dm ** -0.5, gate_cap=15.0))
+            if name == "prefill":
+                rec(tag + "_prefill", sec, flops=4.0 * T * Hm * dm * em)
+            else:
+                rec(tag + "_decode", sec, bytes_=2.0 * batch * Hm * dm * em * 4)
+    # ---- norm and activation ------------------------------------------------------------------------------------------
+    for name, T in (("prefill", prompt_len), ("decode", batch)):
+        res = torch.randn(T, W, device=device)
+        y = torch.randn(T, W, device=device, dtype=bf)
+        w = [torch.randn(W, device=device, dtype=bf) for _ in range(4)]
+        sec = timed(lambda: mops.residual_layer_norm(res, y=y, post=(w[0], w[1]), pre=(w[2], w[3])))
+        x16, r16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
+        lsec = timed(lambda: ops.fused_add_rms_norm(x16, r16, w[0], 1e-5))
+        rec("residual_layer_norm_" + name, sec, bytes_=T * W * (4 + 4 + 2 + 2),
+            like={"kernel": "fused_add_rms_norm", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * W * 8 / lsec / HBM, 3)})
+        gu = torch.randn(T, 2 * ff, device=device, dtype=bf)
+        sec = timed(lambda: mops.act_and_mul(gu, mops.ACT_GELU_TANH))
+        lo = torch.empty(T, ff, device=device, dtype=bf)
+        lsec = timed(lambda: ops.silu_and_mul(lo, gu))
+        rec("act_and_mul_" + name, sec, bytes_=T * ff * 6,
+            like={"kernel": "silu_and_mul", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * ff * 6 / lsec / HBM, 3)})
+    return out
+
+
+def main(args) -> int:
+    from . import _lib
+    from .fatudra import FatudraConfig, FatudraForCausalLM
+    from .model import LlamaConfig, LlamaForCausalLM
+    _lib.lib()
+    _lib.mixers_lib()
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    prompt_len, batch, ctx = args.mixers_prompt, args.batch, args.ctx
+    result = {"metric": "fatudra_vs_llama_bf16_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "n_gpus": 1, "layers": LAYERS, "sizes": {}}
+    with torch.no_grad():
+        for name, s in SIZES.items():
+            if args.mixers_size and name != args.mixers_size:
+                continue
+            t0 = time.time()
+            fat = FatudraForCausalLM(FatudraConfig.from_dict(fatudra_config(s)), torch.bfloat16).init_synthetic(device)
+            r = {"fatudra": model_throughput(fat, prompt_len, batch, ctx, device, VOCAB)}
+            del fat
+            lc = LlamaConfig(hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=LAYERS,
+                             num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=VOCAB,
+                             max_position_embeddings=max(8192, prompt_len + 16))
+            llama = LlamaForCausalLM(lc, None, torch.bfloat16).init_synthetic(device)
+            llama.use_fused_decode = False
+            r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
+            del llama
+            r["kernels"] = kernel_section(s, prompt_len, batch, ctx, device)
+            r["seconds"] = round(time.time() - t0, 1)
+            result["sizes"][name] = r
+            torch.cuda.empty_cache()
+    print(json.dumps(result), flush=True)
+    return 0

@@ -151,6 +151,29 @@ __global__ __launch_bounds__(256) void distance_bias_attention_kernel(
   }
 }
 
+// biased_attention_fast.hip
+struct DBAParams {
+  uint16_t* out;
+  const uint16_t* q;
+  const uint16_t* gate;
+  const uint16_t* k_cache;
+  const uint16_t* v_cache;
+  const int32_t* block_tables;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* ctx_len;
+  const int32_t* seq_of_token;
+  const float* bias_lut;
+  int64_t out_stride, q_stride, gate_stride, num_blocks;
+  int max_blocks, block_size, heads, kv_heads, dim, vdim, lut_len, temp_every, min_len;
+  float scale, temp_coef, out_scale;
+};
+bool dba_prefill_supported(int dim, int vdim);
+bool dba_decode_supported(int heads, int kv_heads, int dim, int vdim);
+void dba_prefill_launch(const DBAParams& p, int max_q_len, int num_seqs, hipStream_t st);
+void dba_decode_launch(const DBAParams& p, int64_t num_tokens, hipStream_t st);
+constexpr int DBA_MFMA_MIN_LEN = 8;     // segments at least this long go to the matrix-core kernel
+
 }  // namespace aphro
 
 using namespace aphro;
@@ -175,9 +198,10 @@ extern "C" int aphro_paged_kv_write(void* k_cache, void* v_cache, const void* k,
 extern "C" int aphro_distance_bias_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
                                              int64_t gate_stride, const void* k_cache, const void* v_cache,
                                              const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size,
-                                             const int32_t* q_start, const int32_t* ctx_len, const int32_t* seq_of_token,
-                                             int64_t num_tokens, int num_seqs, int heads, int kv_heads, int dim, int vdim,
-                                             float scale, const float* bias_lut, int lut_len, float temp_coef, int temp_every,
+                                             const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                                             const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int min_q_len,
+                                             int max_q_len, int heads, int kv_heads, int dim, int vdim, float scale,
+                                             const float* bias_lut, int lut_len, float temp_coef, int temp_every,
                                              float out_scale, int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && q && k_cache && v_cache && block_tables && q_start && ctx_len && seq_of_token,
@@ -191,6 +215,32 @@ extern "C" int aphro_distance_bias_attention(void* out, int64_t out_stride, cons
               "distance_bias_attention: row strides smaller than the rows");
   APHRO_CHECK(!bias_lut || lut_len > 0, "distance_bias_attention: empty bias table");
   APHRO_CHECK(temp_coef == 0.f || temp_every > 0, "distance_bias_attention: temp_every must be positive");
+  // bf16 with 16-byte-aligned rows: the matrix-core kernel for the long segments, the shared-key kernel for the rest
+  if (dtype == APHRO_BF16 && q_len && max_q_len >= min_q_len && min_q_len > 0 && ((uintptr_t)q & 15) == 0 && (q_stride & 7) == 0) {
+    DBAParams p;
+    p.out = (uint16_t*)out; p.q = (const uint16_t*)q; p.gate = (const uint16_t*)gate;
+    p.k_cache = (const uint16_t*)k_cache; p.v_cache = (const uint16_t*)v_cache;
+    p.block_tables = block_tables; p.q_start = q_start; p.q_len = q_len; p.ctx_len = ctx_len; p.seq_of_token = seq_of_token;
+    p.bias_lut = bias_lut; p.out_stride = out_stride; p.q_stride = q_stride; p.gate_stride = gate_stride; p.num_blocks = num_blocks;
+    p.max_blocks = max_blocks; p.block_size = block_size; p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim;
+    p.lut_len = lut_len; p.temp_every = temp_every; p.scale = scale; p.temp_coef = temp_coef; p.out_scale = out_scale;
+    const bool pf = dba_prefill_supported(dim, vdim) && max_q_len >= DBA_MFMA_MIN_LEN;
+    const bool dc = dba_decode_supported(heads, kv_heads, dim, vdim);
+    const bool all_long = min_q_len >= DBA_MFMA_MIN_LEN;
+    if (pf && (all_long || dc)) {
+      p.min_len = DBA_MFMA_MIN_LEN;
+      dba_prefill_launch(p, max_q_len, num_seqs, (hipStream_t)stream);
+      if (!all_long) dba_decode_launch(p, num_tokens, (hipStream_t)stream);
+      APHRO_LAUNCH_CHECK();
+      return APHRO_OK;
+    }
+    if (dc) {
+      p.min_len = 0x7fffffff;
+      dba_decode_launch(p, num_tokens, (hipStream_t)stream);
+      APHRO_LAUNCH_CHECK();
+      return APHRO_OK;
+    }
+  }
   const dim3 grid((unsigned)num_tokens, (unsigned)heads);
   const int epl = (vdim + 63) / 64;
 #define DBA_LAUNCH(EPL)                                                                                                   \

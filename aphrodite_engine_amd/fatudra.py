@@ -69,7 +69,16 @@ class FatudraConfig:
 def _linear(width_in: int, outs: List[int], dtype, bias: bool, prefix: str):
     from .loader import merged_plan
     from .model import QuantLinear
-    return QuantLinear(width_in, outs, None, dtype, prefix=prefix, plan=merged_plan(outs), bias=bias)
+    lin = QuantLinear(width_in, outs, None, dtype, prefix=prefix, plan=merged_plan(outs), bias=bias)
+    lin.weight.data.zero_()
+    return lin
+
+
+def _padded(splits: List[int]) -> List[int]:
+    """A last, never-loaded all-zero partition that makes the fused product's rows a multiple of 16 bytes: the column
+    slices handed to the kernels then keep 16-byte-aligned rows whenever their own offsets do."""
+    pad = -sum(splits) % 8
+    return splits + [pad] if pad else list(splits)
 
 
 class ParallelMixer(nn.Module):
@@ -90,6 +99,7 @@ class ParallelMixer(nn.Module):
         self.memory = OuterProductMemory(mops.MEMORY_DECAY, Hr, dr, er, decay=[float(x) for x in R["decay"]])
         self.splits = [H * d, G * d, G * e, H, Hr * dr, Hr * dr, Hr * er, Hr * er]
         self.names = ["left.q", "left.k", "left.v", "left.g", "right.q", "right.k", "right.v", "right.g"]
+        self.splits = _padded(self.splits)
         self.in_proj = _linear(width, self.splits, dtype, True, prefix + "in_proj")
         self.left_out, self.right_out = H * e, Hr * er
         self.out_proj = _linear(self.left_out + self.right_out, [width], dtype, False, prefix + "out_proj")
@@ -105,7 +115,7 @@ class ParallelMixer(nn.Module):
         self.out_bias = (self.left_out_bias.float() * self.left_scale).contiguous()
 
     def forward(self, h: torch.Tensor, caches, batch: StepBatch) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-        lq, lk, lv, lg, rq, rk, rv, rg = self.in_proj(h).split(self.splits, dim=-1)
+        lq, lk, lv, lg, rq, rk, rv, rg = self.in_proj(h).split(self.splits, dim=-1)[:8]
         cat = torch.empty(h.shape[0], self.left_out + self.right_out, dtype=h.dtype, device=h.device)
         self.attn(cat[:, :self.left_out], lq, lk, lv, lg, caches[0], batch, out_scale=self.left_scale)
         o = self.memory(rq, rk, rv, caches[1], batch)
@@ -123,6 +133,7 @@ class MLSTMMixer(nn.Module):
         self.memory = OuterProductMemory(mops.MEMORY_MLSTM, H, d, e, q_scale=d ** -0.5, gate_cap=float(mc["gate_cap"]))
         self.splits = [H * d, H * d, H * e, H * e, H, H]
         self.names = ["q", "k", "v", "g", "i", "f"]
+        self.splits = _padded(self.splits)
         self.in_proj = _linear(width, self.splits, dtype, True, prefix + "in_proj")
         self.out_proj = _linear(H * e, [width], dtype, False, prefix + "out_proj")
         self.norm = nn.Parameter(torch.ones(H * e, dtype=dtype), requires_grad=False)
@@ -134,7 +145,7 @@ class MLSTMMixer(nn.Module):
         pass
 
     def forward(self, h: torch.Tensor, caches, batch: StepBatch) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-        q, k, v, g, gi, gf = self.in_proj(h).split(self.splits, dim=-1)
+        q, k, v, g, gi, gf = self.in_proj(h).split(self.splits, dim=-1)[:6]
         o = self.memory(q, k, v, caches[0], batch, gate_i=gi, gate_f=gf)
         normed = torch.empty(h.shape[0], o.shape[1], dtype=h.dtype, device=h.device)
         mops.gated_group_rms_norm(normed, o, self.norm, g, self.vdim, self.eps)
@@ -315,9 +326,12 @@ class FatudraForCausalLM(nn.Module):
         raise ValueError(f"unexpected tensor {name!r}")
 
     @torch.no_grad()
-    def init_synthetic(self, device, seed: int = 0):
+    def init_synthetic(self, device, seed: int = 0, bias_rows: int = 32):
         """Random weights of the checkpoint's scale on the device (benchmarks, tests)."""
         g = torch.Generator(device="cpu").manual_seed(seed)
+        for layer in self.layers:
+            if isinstance(layer.mix, ParallelMixer):
+                layer.mix.attn.rel = nn.Parameter(torch.zeros(bias_rows, layer.mix.attn.heads), requires_grad=False)
         self.to(device)
         for name, p in self.named_parameters():
             if p.dim() >= 2:

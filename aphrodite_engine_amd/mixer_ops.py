@@ -145,13 +145,17 @@ def paged_kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, k: torch.Tensor
 
 
 def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor,
-                            v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
-                            seq_of_token: torch.Tensor, heads: int, scale: float, bias_lut: Optional[torch.Tensor],
-                            temp_coef: float = 0.0, temp_every: int = 1, out_scale: float = 1.0) -> None:
+                            v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                            ctx_len: torch.Tensor, seq_of_token: torch.Tensor, q_len_range, heads: int, scale: float,
+                            bias_lut: Optional[torch.Tensor], temp_coef: float = 0.0, temp_every: int = 1,
+                            out_scale: float = 1.0) -> None:
     """Causal attention of a batch of segments over the paged cache, written into ``out`` [T, heads * e] (dense rows, any
     row stride).  q [T, heads * d]; gate [T, heads] raw (sigmoid inside) or None; bias_lut fp32 [heads, L] indexed by
-    min(distance, L - 1) or None."""
-    _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, ctx_len, seq_of_token, bias_lut)
+    min(distance, L - 1) or None.  ``q_len_range``: (shortest, longest) segment of the batch, known on the host -- it
+    chooses between the matrix-core kernel for prompt portions and the shared-key kernel for single tokens."""
+    _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, q_len, ctx_len, seq_of_token, bias_lut)
+    lo, hi = int(q_len_range[0]), int(q_len_range[1])
+    _need(0 < lo <= hi, "distance_bias_attention: q_len_range (shortest, longest)")
     nb, bs, G, d = k_cache.shape
     e = v_cache.shape[3]
     T = q.shape[0]
@@ -162,6 +166,7 @@ def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[t
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.is_contiguous(),
           "distance_bias_attention: block_tables int32 [S, max_blocks]")
     _i32(q_start, S, "q_start")
+    _i32(q_len, S, "q_len")
     _i32(ctx_len, S, "ctx_len")
     _i32(seq_of_token, T, "seq_of_token")
     gs = 0
@@ -175,8 +180,8 @@ def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[t
         L = bias_lut.shape[1]
     check(_lib.mixers_lib().aphro_distance_bias_attention(
         out.data_ptr(), _rows(out, heads * e, "out"), q.data_ptr(), _rows(q, heads * d, "q"), _p(gate), gs, k_cache.data_ptr(),
-        v_cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(),
-        seq_of_token.data_ptr(), T, S, heads, G, d, e, float(scale), _p(bias_lut), L, float(temp_coef), int(temp_every),
+        v_cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(),
+        ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, lo, hi, heads, G, d, e, float(scale), _p(bias_lut), L, float(temp_coef), int(temp_every),
         float(out_scale), _dt(q), _stream()), "distance_bias_attention")
 
 

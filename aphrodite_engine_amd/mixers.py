@@ -96,9 +96,9 @@ class DistanceBiasAttention(nn.Module):
     def forward(self, out: torch.Tensor, q, k, v, gate, cache, batch: StepBatch, out_scale: float = 1.0) -> None:
         k_cache, v_cache = cache
         mops.paged_kv_write(k_cache, v_cache, k, v, batch.slot_mapping)
-        mops.distance_bias_attention(out, q, gate, k_cache, v_cache, batch.block_tables, batch.q_start, batch.ctx_len,
-                                     batch.seq_of_token, self.heads, self.scale, self.bias_lut, self.temp_coef,
-                                     self.temp_every, out_scale)
+        mops.distance_bias_attention(out, q, gate, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len,
+                                     batch.ctx_len, batch.seq_of_token, (min(batch.q_lens), max(batch.q_lens)), self.heads,
+                                     self.scale, self.bias_lut, self.temp_coef, self.temp_every, out_scale)
 
 
 class OuterProductMemory(nn.Module):

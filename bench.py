@@ -95,6 +95,12 @@ def parse_args():
                     help="N > 1, replicas: skip the tensor-parallel section (TP = N timing, overlap A/B, all-reduce latencies)")
     ap.add_argument("--tp-child", action="store_true", help="(internal) the tensor-parallel section of an N > 1 run, in its own processes")
     ap.add_argument("--layers", type=int, default=0, help="debug only: fewer layers (marks the line invalid)")
+    ap.add_argument("--mixers", action="store_true",
+                    help="instead of the default workload: a Fatudra stack (biased attention + decay memory + mLSTM layers) beside a "
+                         "Llama stack of equal size, bf16, prefill (--mixers-prompt tokens) and decode (--batch x --ctx), and every "
+                         "mixer kernel alone against its roofline (aphrodite_engine_amd/bench_mixers.py); one JSON line of its own")
+    ap.add_argument("--mixers-prompt", type=int, default=4096)
+    ap.add_argument("--mixers-size", default="", choices=["", "w2048", "w4096"])
     return ap.parse_args()
 
 
@@ -1052,6 +1058,9 @@ def main():
         return tp_child_main(args)
     if os.environ.get("APHRO_BENCH_DRY_CPU") == "1":
         return main_dry_cpu(args)
+    if args.mixers:
+        from aphrodite_engine_amd import bench_mixers
+        return bench_mixers.main(args)
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

@@ -65,13 +65,17 @@ int aphro_paged_kv_write(void* k_cache, void* v_cache, const void* k, int64_t k_
  *   out[t, h, :] = out_scale * sigmoid(gate[t, h]) * sum_j softmax_j(score) v_j     (gate NULL: no gate)
  * q [T, heads * dim] (row stride), gate [T, heads] (row stride) and out [T, heads * vdim] (row stride) of `dtype`;
  * bias_lut fp32 [heads, lut_len] (NULL: no bias); block_tables int32 [num_seqs, max_blocks]; seq_of_token int32 [T].
- * Query head h reads key/value head h / (heads / kv_heads). */
+ * Query head h reads key/value head h / (heads / kv_heads).  q_len int32 [num_seqs] with its host-side minimum and
+ * maximum choose the kernels: bf16 segments of 8 rows or more run on the matrix cores (dim, vdim in {32, 64, 96, 128}),
+ * shorter ones on a kernel that reads each key once for all query heads of its kv head (dim, vdim multiples of 8, at most
+ * 256, 1 / 2 / 4 / 8 query heads per kv head); every other case -- and fp32 -- runs the scalar fp32 kernel. */
 int aphro_distance_bias_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
                                   int64_t gate_stride, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                   int max_blocks, int64_t num_blocks, int block_size, const int32_t* q_start,
-                                  const int32_t* ctx_len, const int32_t* seq_of_token, int64_t num_tokens, int num_seqs,
-                                  int heads, int kv_heads, int dim, int vdim, float scale, const float* bias_lut, int lut_len,
-                                  float temp_coef, int temp_every, float out_scale, int dtype, void* stream);
+                                  const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token,
+                                  int64_t num_tokens, int num_seqs, int min_q_len, int max_q_len, int heads, int kv_heads,
+                                  int dim, int vdim, float scale, const float* bias_lut, int lut_len, float temp_coef,
+                                  int temp_every, float out_scale, int dtype, void* stream);
 
 /* Gated outer-product memory, one state per (slot, head):  S <- a_t S + b_t k_t v_t^T,  o_t = S^T q_t  [/ normaliser].
  *   mode 0 (decay linear attention): q, k, v = silu(raw); a_t = decay[h], b_t = 1.

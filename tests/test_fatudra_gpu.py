@@ -125,7 +125,8 @@ def run_attention(mops, pg, qs, ctx, H, scale, lut, coef, every, dtype, gate=Non
     e = pg.vc.shape[3]
     out = torch.full((q.shape[0], H * e + 3), 7.0, dtype=dtype, device=DEV)
     mops.distance_bias_attention(out[:, :H * e], q, None if gate is None else dev(gate, dtype), pg.kc, pg.vc, bt,
-                                 i32(starts), i32(ctx), i32(seq_of), H, scale, lut, coef, every, out_scale)
+                                 i32(starts), i32(lens), i32(ctx), i32(seq_of), (min(lens), max(lens)), H, scale, lut, coef, every,
+                                 out_scale)
     assert float((out[:, H * e:] - 7.0).abs().sum()) == 0
     return out[:, :H * e].float().cpu().numpy().reshape(-1, H, e)
 
