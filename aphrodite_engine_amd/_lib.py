@@ -174,8 +174,8 @@ MIXERS_SIGNATURES = {
     "aphro_gated_group_rms_norm": (I, [P, L, P, P, P, L, L, I, I, F, F, I, P]),
     "aphro_paged_kv_write": (I, [P, P, P, L, P, L, P, L, I, I, I, L, I, P]),
     "aphro_distance_bias_attention": (I, [P, L, P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, F, P, I, F,
-                                          I, F, I, P]),
-    "aphro_outer_memory_scan": (I, [P, P, L, P, L, P, L, P, P, L, P, P, P, P, I, P, P, P, I, L, I, I, I, I, P, F, F, I, P]),
+                                          I, F, I, P, L, I, P]),
+    "aphro_outer_memory_scan": (I, [P, P, L, P, L, P, L, P, P, L, P, P, P, P, I, P, P, P, I, L, I, I, I, I, P, F, F, I, I, P]),
 }
 
 OK = 0

@@ -108,7 +108,8 @@ def kernel_section(s, prompt_len, batch, ctx, device):
         gate = torch.randn(T, H, device=device, dtype=bf)
         o = torch.empty(T, H * d, device=device, dtype=bf)
         sec = timed(lambda: mops.distance_bias_attention(o, q, gate, kc, vc, b.block_tables, b.q_start, b.q_len, b.ctx_len,
-                                                         b.seq_of_token, (min(b.q_lens), max(b.q_lens)), H, att.scale, att.bias_lut, att.temp_coef, att.temp_every))
+                                                         b.seq_of_token, (min(b.q_lens), max(b.q_lens)), H, att.scale, att.bias_lut, att.temp_coef, att.temp_every,
+                                                         max_kv_len=max(c + n for c, n in zip(b.ctx_lens, b.q_lens))))
         if name == "prefill":
             flops = 4.0 * d * H * T * (T + 1) / 2
             k = torch.randn(T, G, d, device=device, dtype=bf)
@@ -138,7 +139,8 @@ def kernel_section(s, prompt_len, batch, ctx, device):
             v = torch.randn(T, Hm * em, device=device, dtype=bf)
             gi, gf = torch.randn(T, Hm, device=device, dtype=bf), torch.randn(T, Hm, device=device, dtype=bf) + 3
             sec = timed(lambda: mops.outer_memory_scan(q, k, v, state, b.state_slots, b.q_start, b.q_len, b.ctx_len, Hm, mode,
-                                                       decay=decay, gate_i=gi, gate_f=gf, q_scale=dm ** -0.5, gate_cap=15.0))
+                                                       decay=decay, gate_i=gi, gate_f=gf, q_scale=dm ** -0.5, gate_cap=15.0,
+                                                       max_q_len=max(b.q_lens)))
             if name == "prefill":
                 rec(tag + "_prefill", sec, flops=4.0 * T * Hm * dm * em)
             else:

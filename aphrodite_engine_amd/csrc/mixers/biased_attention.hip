@@ -167,11 +167,14 @@ struct DBAParams {
   int64_t out_stride, q_stride, gate_stride, num_blocks;
   int max_blocks, block_size, heads, kv_heads, dim, vdim, lut_len, temp_every, min_len;
   float scale, temp_coef, out_scale;
+  float* ws;
+  int bs_shift;
 };
 bool dba_prefill_supported(int dim, int vdim);
 bool dba_decode_supported(int heads, int kv_heads, int dim, int vdim);
 void dba_prefill_launch(const DBAParams& p, int max_q_len, int num_seqs, hipStream_t st);
-void dba_decode_launch(const DBAParams& p, int64_t num_tokens, hipStream_t st);
+void dba_decode_launch(const DBAParams& p, int64_t num_tokens, int nsplit, hipStream_t st);
+int dba_decode_splits(int64_t num_tokens, int kv_heads, int max_kv_len, int64_t ws_floats, int heads, int vdim);
 constexpr int DBA_MFMA_MIN_LEN = 8;     // segments at least this long go to the matrix-core kernel
 
 }  // namespace aphro
@@ -202,7 +205,8 @@ extern "C" int aphro_distance_bias_attention(void* out, int64_t out_stride, cons
                                              const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int min_q_len,
                                              int max_q_len, int heads, int kv_heads, int dim, int vdim, float scale,
                                              const float* bias_lut, int lut_len, float temp_coef, int temp_every,
-                                             float out_scale, int dtype, void* stream) {
+                                             float out_scale, int max_kv_len, float* workspace, int64_t workspace_floats,
+                                             int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && q && k_cache && v_cache && block_tables && q_start && ctx_len && seq_of_token,
               "distance_bias_attention: null argument");
@@ -224,19 +228,24 @@ extern "C" int aphro_distance_bias_attention(void* out, int64_t out_stride, cons
     p.bias_lut = bias_lut; p.out_stride = out_stride; p.q_stride = q_stride; p.gate_stride = gate_stride; p.num_blocks = num_blocks;
     p.max_blocks = max_blocks; p.block_size = block_size; p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim;
     p.lut_len = lut_len; p.temp_every = temp_every; p.scale = scale; p.temp_coef = temp_coef; p.out_scale = out_scale;
+    p.ws = workspace;
+    p.bs_shift = -1;
+    for (int sft = 0; sft < 20; ++sft)
+      if ((1 << sft) == block_size) p.bs_shift = sft;
+    const int nsplit = workspace ? dba_decode_splits(num_tokens, kv_heads, max_kv_len, workspace_floats, heads, vdim) : 1;
     const bool pf = dba_prefill_supported(dim, vdim) && max_q_len >= DBA_MFMA_MIN_LEN;
     const bool dc = dba_decode_supported(heads, kv_heads, dim, vdim);
     const bool all_long = min_q_len >= DBA_MFMA_MIN_LEN;
     if (pf && (all_long || dc)) {
       p.min_len = DBA_MFMA_MIN_LEN;
       dba_prefill_launch(p, max_q_len, num_seqs, (hipStream_t)stream);
-      if (!all_long) dba_decode_launch(p, num_tokens, (hipStream_t)stream);
+      if (!all_long) dba_decode_launch(p, num_tokens, nsplit, (hipStream_t)stream);
       APHRO_LAUNCH_CHECK();
       return APHRO_OK;
     }
     if (dc) {
       p.min_len = 0x7fffffff;
-      dba_decode_launch(p, num_tokens, (hipStream_t)stream);
+      dba_decode_launch(p, num_tokens, nsplit, (hipStream_t)stream);
       APHRO_LAUNCH_CHECK();
       return APHRO_OK;
     }

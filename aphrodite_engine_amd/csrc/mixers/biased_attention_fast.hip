@@ -2,17 +2,20 @@
 // the path of sizes these do not tile):
 //
 //  * dba_prefill_kernel<DK, DV>: segments of >= DBA_MFMA_MIN_LEN rows.  A workgroup of four waves owns 64 consecutive
-//    query rows of one (segment, head), 16 rows per wave, and walks the visible keys 32 at a time: the K rows and V rows of
-//    the tile come from the paged cache with 16-byte loads into LDS (K chunk-swizzled, V transposed), together with the 95
-//    bias values the tile can need (the table is indexed by distance, and a 64 x 32 tile spans 95 distances).
+//    query rows of one (segment, head), 16 rows per wave, and walks the visible keys 64 at a time: the K rows and V rows of
+//    the tile come from the paged cache with 16-byte loads into LDS (K chunk-swizzled, V transposed), together with the 127
+//    bias values the tile can need (the table is indexed by distance, and a 64 x 64 tile spans 127 distances); the next
+//    tile's cache rows are fetched into registers while the current tile's products run.
 //    S^T = K Q^T on v_mfma_f32_16x16x32_bf16, so that the probabilities come out in the B-operand layout of O^T = V^T P^T
 //    (keys of the two 16-key halves interleaved per lane group, V fragments read in the same order); temperature, bias,
 //    mask and the online softmax are fp32 on the accumulator registers.
 //  * dba_decode_kernel<QH, CHL>: the other rows (single decoded tokens, short portions), one workgroup per (row, kv head)
 //    serving all QH query heads of that kv head from one pass over the keys.  A key row is read by 2^CHL lanes x 16 bytes,
 //    64 / 2^CHL keys per load instruction (fully coalesced); the partial dot products fold over the lanes of a key with
-//    DPP shuffles; scores and probabilities stay in that layout (16 keys x QH per lane), which is also the layout the V
-//    pass wants, so nothing is redistributed.  Four waves split the 64-key tiles; partial (max, sum, acc) merge in LDS.
+//    DPP shuffles; scores and probabilities stay in that layout (4 keys x QH per lane and step), which is also the layout
+//    the V pass wants, so nothing is redistributed; K and V of a step are fetched together.  Four waves take the steps
+//    round-robin and merge their (max, sum, acc) in LDS; long key ranges are also split over workgroups (grid z), whose
+//    partial results dba_merge_kernel combines.
 #include "mixers_common.h"
 
 namespace aphro {
@@ -32,21 +35,101 @@ struct DBAParams {          // (declared alike in biased_attention.hip, which fi
   int64_t out_stride, q_stride, gate_stride, num_blocks;
   int max_blocks, block_size, heads, kv_heads, dim, vdim, lut_len, temp_every, min_len;
   float scale, temp_coef, out_scale;
+  float* ws;          // decode split partials [T, heads, nsplit, 2 + vdim]
+  int bs_shift;       // log2(block_size), or -1 when it is no power of two
 };
+
+// row of key `key` in the token-major cache ([block, offset] -> block * block_size + offset), following the block table
+__device__ __forceinline__ int dba_slot(const DBAParams& p, const int32_t* bt, int key) {
+  int blk, off;
+  if (p.bs_shift >= 0) {
+    blk = bt[key >> p.bs_shift];
+    off = key & (p.block_size - 1);
+  } else {
+    blk = bt[key / p.block_size];
+    off = key % p.block_size;
+  }
+  if (blk < 0 || blk >= p.num_blocks) blk = 0;             // never read outside the pool
+  return blk * p.block_size + off;
+}
 
 __device__ __forceinline__ float dba_temp(const DBAParams& p, int pos) {
   return p.temp_coef != 0.f ? 1.0f + p.temp_coef * logf((float)((pos + 1) / p.temp_every + 1)) : 1.0f;
 }
 
-constexpr int PF_BM = 64, PF_BN = 32, PF_VT = 36;
+constexpr int PF_BM = 64, PF_BN = 64, PF_VT = PF_BN + 4;
+
+// One thread's share of a key tile on its way from the cache to LDS: K chunks (one key, 16 bytes) and V chunk pairs (two
+// neighbouring keys, so that the transposed LDS stores are whole dwords).
+template <int DK, int DV>
+struct PFStage {
+  static constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  static constexpr int KI = (PF_BN * NCHK + 255) / 256, VI = (PF_BN / 2 * NCHV + 255) / 256;
+  u16x8 k[KI], v0[VI], v1[VI];
+};
+
+template <int DK, int DV>
+__device__ __forceinline__ void pf_load(PFStage<DK, DV>& st, const DBAParams& p, const int32_t* bt, int kvh, int t0, int nk) {
+  constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  const int64_t krow = (int64_t)p.kv_heads * DK, vrow = (int64_t)p.kv_heads * DV;
+#pragma unroll
+  for (int it = 0; it < PFStage<DK, DV>::KI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < PF_BN * NCHK) {
+      const int tok = i / NCHK, ch = i % NCHK;
+      const int key = min(t0 + tok, nk - 1);
+      st.k[it] = *reinterpret_cast<const u16x8*>(p.k_cache + (int64_t)dba_slot(p, bt, key) * krow + kvh * DK + 8 * ch);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < PFStage<DK, DV>::VI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < PF_BN / 2 * NCHV) {
+      const int tp = i / NCHV, ch = i % NCHV;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int key = min(t0 + 2 * tp + half, nk - 1);
+        u16x8 vv = *reinterpret_cast<const u16x8*>(p.v_cache + (int64_t)dba_slot(p, bt, key) * vrow + kvh * DV + 8 * ch);
+        if (t0 + 2 * tp + half >= nk) vv = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (half == 0) st.v0[it] = vv;
+        else st.v1[it] = vv;
+      }
+    }
+  }
+}
+
+template <int DK, int DV>
+__device__ __forceinline__ void pf_store(const PFStage<DK, DV>& st, uint16_t* k_lds, uint16_t* vt_lds) {
+  constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  constexpr int SWZ = (NCHK & -NCHK) - 1;
+#pragma unroll
+  for (int it = 0; it < PFStage<DK, DV>::KI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < PF_BN * NCHK) {
+      const int tok = i / NCHK, ch = i % NCHK;
+      *reinterpret_cast<u16x8*>(&k_lds[tok * DK + 8 * (ch ^ (tok & SWZ))]) = st.k[it];
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < PFStage<DK, DV>::VI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < PF_BN / 2 * NCHV) {
+      const int tp = i / NCHV, ch = i % NCHV;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<uint32_t*>(&vt_lds[(8 * ch + j) * PF_VT + 2 * tp]) = (uint32_t)st.v0[it][j] | ((uint32_t)st.v1[it][j] << 16);
+    }
+  }
+}
 
 template <int DK, int DV>
 __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
-  constexpr int NCHK = DK / 8, NCHV = DV / 8, NKS = DK / 32, NDT = DV / 16;
+  constexpr int NCHK = DK / 8, NKS = DK / 32, NDT = DV / 16, NH = PF_BN / 16, NPK = PF_BN / 32;
   constexpr int SWZ = (NCHK & -NCHK) - 1;
+  constexpr int NWIN = PF_BM + PF_BN - 1;
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[PF_BN * DK];
   __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DV * PF_VT];
-  __shared__ float bias_win[96];
+  __shared__ float bias_win[NWIN + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
   const int head = blockIdx.y, seq = blockIdx.z;
   const int len = p.q_len[seq];
@@ -60,7 +143,8 @@ __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
   const int qrow = q0 + 16 * wave + c;
   const bool qvalid = qrow < len;
   const int qpos = ctx + qrow;
-  const float qs = p.scale * dba_temp(p, qpos);
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float qs = p.scale * dba_temp(p, qpos) * LOG2E;     // scores in units of ln 2: the exponentials are exp2
   u32x4 qf[NKS];
   {
     const uint16_t* qp = p.q + (int64_t)(s0 + min(qrow, len - 1)) * p.q_stride + head * DK;
@@ -74,44 +158,27 @@ __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
   const float* lut = p.bias_lut ? p.bias_lut + (int64_t)head * p.lut_len : nullptr;
   const int nk = ctx + min(len, q0 + PF_BM);               // keys the tile's last row sees
-  const int64_t krow = (int64_t)p.kv_heads * DK, vrow = (int64_t)p.kv_heads * DV;
 
+  PFStage<DK, DV> st;
+  pf_load<DK, DV>(st, p, bt, kvh, 0, nk);
   for (int t0 = 0; t0 < nk; t0 += PF_BN) {
-    __syncthreads();
-    for (int i = threadIdx.x; i < PF_BN * NCHK; i += 256) {
-      const int tok = i / NCHK, ch = i % NCHK;
-      const int key = min(t0 + tok, nk - 1);
-      int blk = bt[key / p.block_size];
-      if (blk < 0 || blk >= p.num_blocks) blk = 0;
-      const u16x8 kk = *reinterpret_cast<const u16x8*>(p.k_cache + ((int64_t)blk * p.block_size + key % p.block_size) * krow +
-                                                       kvh * DK + 8 * ch);
-      *reinterpret_cast<u16x8*>(&k_lds[tok * DK + 8 * (ch ^ (tok & SWZ))]) = kk;
-    }
-    for (int i = threadIdx.x; i < PF_BN * NCHV; i += 256) {
-      const int tok = i / NCHV, ch = i % NCHV;
-      const int key = min(t0 + tok, nk - 1);
-      int blk = bt[key / p.block_size];
-      if (blk < 0 || blk >= p.num_blocks) blk = 0;
-      u16x8 vv = *reinterpret_cast<const u16x8*>(p.v_cache + ((int64_t)blk * p.block_size + key % p.block_size) * vrow +
-                                                 kvh * DV + 8 * ch);
-      if (t0 + tok >= nk) vv = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) vt_lds[(8 * ch + j) * PF_VT + tok] = vv[j];
-    }
+    __syncthreads();                                        // the previous tile is consumed
+    pf_store<DK, DV>(st, k_lds, vt_lds);
     const int dmin = ctx + q0 - t0 - (PF_BN - 1);           // distance of (first row, last key of the tile)
-    if (threadIdx.x < 95) {
+    if (threadIdx.x < NWIN) {
       float b = 0.f;
       if (lut) {
         const int dist = dmin + (int)threadIdx.x;
-        b = lut[dist < 0 ? 0 : (dist < p.lut_len ? dist : p.lut_len - 1)];
+        b = lut[dist < 0 ? 0 : (dist < p.lut_len ? dist : p.lut_len - 1)] * LOG2E;
       }
       bias_win[threadIdx.x] = b;
     }
     __syncthreads();
+    if (t0 + PF_BN < nk) pf_load<DK, DV>(st, p, bt, kvh, t0 + PF_BN, nk);      // in flight during this tile's products
     if (t0 > ctx + q0 + 16 * wave + 15) continue;           // every key of the tile is ahead of the wave's rows
-    f32x4 s[2];
+    f32x4 s[NH];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < NH; ++h) {
       s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
       const int tok = 16 * h + c;
 #pragma unroll
@@ -121,44 +188,48 @@ __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
         s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
       }
     }
-    float pv[2][4];
+    float pv[NH][4];
     float mx = -1e30f;
+    const float* bw = &bias_win[qpos - t0 - dmin - 4 * g];  // bias of (this row, key t0 + 4 g); keys count downwards
+    const bool diag = t0 + PF_BN - 1 > ctx + q0 + 16 * wave; // some key of the tile is ahead of some row of the wave
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < NH; ++h)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int key = t0 + 16 * h + 4 * g + r;
-        float xv = s[h][r] * qs + bias_win[qpos - key - dmin];
-        xv = key <= qpos ? xv : -1e30f;
+        float xv = s[h][r] * qs + bw[-(16 * h + r)];
+        if (diag) xv = t0 + 16 * h + 4 * g + r <= qpos ? xv : -1e30f;
         pv[h][r] = xv;
         mx = fmaxf(mx, xv);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __expf(m_run - m_new);
+    const float m_new = fmaxf(m_run, mx);                   // finite for every row that is kept: key 0 is visible
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     m_run = m_new;
     float lsum = 0.f;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < NH; ++h)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float e = pv[h][r] > -1e29f ? __expf(pv[h][r] - m_new) : 0.f;
+        const float e = __builtin_amdgcn_exp2f(pv[h][r] - m_new);           // a masked score is 1e30 below: exactly 0
         pv[h][r] = e;
         lsum += e;
       }
     l_run = l_run * alpha + lsum;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[dt] *= alpha;
-    const u32x4 pf = {pack2_16<true>(pv[0][0], pv[0][1]), pack2_16<true>(pv[0][2], pv[0][3]), pack2_16<true>(pv[1][0], pv[1][1]),
-                      pack2_16<true>(pv[1][2], pv[1][3])};
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      const uint16_t* vr = &vt_lds[(16 * dt + c) * PF_VT + 4 * g];
-      const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
-      const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
-      const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
+    for (int pk = 0; pk < NPK; ++pk) {
+      const u32x4 pf = {pack2_16<true>(pv[2 * pk][0], pv[2 * pk][1]), pack2_16<true>(pv[2 * pk][2], pv[2 * pk][3]),
+                        pack2_16<true>(pv[2 * pk + 1][0], pv[2 * pk + 1][1]), pack2_16<true>(pv[2 * pk + 1][2], pv[2 * pk + 1][3])};
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const uint16_t* vr = &vt_lds[(16 * dt + c) * PF_VT + 32 * pk + 4 * g];
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
+      }
     }
   }
   l_run += __shfl_xor(l_run, 16, 64);
@@ -178,7 +249,8 @@ template <int QH, int CHL>
 __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
   constexpr int CH = 1 << CHL;       // lanes per key row (16 bytes each)
   constexpr int KP = 64 / CH;        // keys per load instruction
-  constexpr int NI = CH;             // load instructions per 64-key tile
+  constexpr int NI = 4;              // load instructions per step of the online softmax (few: registers buy occupancy)
+  constexpr int KT = NI * KP;        // keys per step
   __shared__ float merge[4][QH][2 + 8 * CH];
   const int t = blockIdx.x, kvh = blockIdx.y;
   const int seq = p.seq_of_token[t];
@@ -207,20 +279,21 @@ __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[qh][j] = 0.f;
   }
-  const int ntiles = (nkeys + 63) >> 6;
-  for (int tile = wave; tile < ntiles; tile += 4) {
+  const int ntiles = (nkeys + KT - 1) / KT;
+  const int nsplit = gridDim.z, tps = (ntiles + nsplit - 1) / nsplit;
+  const int tile_end = min(ntiles, ((int)blockIdx.z + 1) * tps);
+  for (int tile = (int)blockIdx.z * tps + wave; tile < tile_end; tile += 4) {
     float sc[NI][QH];
-    int64_t voff[NI];
+    u16x8 vv[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int key = tile * 64 + i * KP + kg;
+      const int key = tile * KT + i * KP + kg;
       const bool valid = key < nkeys;
-      int blk = valid ? bt[key / p.block_size] : 0;
-      if (blk < 0 || blk >= p.num_blocks) blk = 0;
-      const int64_t slot = (int64_t)blk * p.block_size + (valid ? key % p.block_size : 0);
-      voff[i] = slot * vrow + kvh * p.vdim + 8 * ck;
+      const int64_t slot = dba_slot(p, bt, valid ? key : 0);
       u16x8 kk = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      vv[i] = kk;
       if (valid && kin) kk = *reinterpret_cast<const u16x8*>(p.k_cache + slot * krow + kvh * p.dim + 8 * ck);
+      if (valid && vin) vv[i] = *reinterpret_cast<const u16x8*>(p.v_cache + slot * vrow + kvh * p.vdim + 8 * ck);
       float kf[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) kf[j] = BFloat::to_f32(kk[j]);
@@ -230,8 +303,7 @@ __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
         float d = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) d += qv[qh][j] * kf[j];
-#pragma unroll
-        for (int o = 1; o < CH; o <<= 1) d += __shfl_xor(d, o, 64);
+        d = group_sum<CHL>(d);
         float b = 0.f;
         if (p.bias_lut && valid) b = p.bias_lut[(int64_t)(kvh * QH + qh) * p.lut_len + (dist < p.lut_len ? dist : p.lut_len - 1)];
         sc[i][qh] = valid ? d * qs + b : -INFINITY;
@@ -244,7 +316,7 @@ __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
       for (int i = 1; i < NI; ++i) mx = fmaxf(mx, sc[i][qh]);
 #pragma unroll
       for (int o = CH; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      const float m_new = fmaxf(m[qh], mx);                // finite: key tile*64 exists
+      const float m_new = fmaxf(m[qh], mx);                // finite: the tile's first key exists
       const float alpha = (m[qh] == -INFINITY) ? 0.f : __expf(m[qh] - m_new);
       m[qh] = m_new;
       float ls = 0.f;
@@ -260,12 +332,9 @@ __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
     }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int key = tile * 64 + i * KP + kg;
-      u16x8 vv = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (key < nkeys && vin) vv = *reinterpret_cast<const u16x8*>(p.v_cache + voff[i]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float vf = BFloat::to_f32(vv[j]);
+        const float vf = BFloat::to_f32(vv[i][j]);
 #pragma unroll
         for (int qh = 0; qh < QH; ++qh) acc[qh][j] += sc[i][qh] * vf;
       }
@@ -303,8 +372,40 @@ __global__ __launch_bounds__(256) void dba_decode_kernel(DBAParams p) {
       o += merge[w][qh][2 + col] * f;
     }
     const int head = kvh * QH + qh;
+    if (nsplit > 1) {                                       // this split's share; dba_merge_kernel finishes the row
+      float* w = p.ws + (((int64_t)t * p.heads + head) * nsplit + blockIdx.z) * (2 + p.vdim);
+      if (col == 0) {
+        w[0] = M;
+        w[1] = L;
+      }
+      w[2 + col] = o;
+      continue;
+    }
     float sig = p.out_scale;
     if (p.gate) sig *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head]));
+    p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(o * sig / L);
+  }
+}
+
+__global__ void dba_merge_kernel(DBAParams p, int nsplit) {
+  const int t = blockIdx.x, head = blockIdx.y;
+  if (p.q_len[p.seq_of_token[t]] >= p.min_len) return;
+  const float* w = p.ws + ((int64_t)t * p.heads + head) * nsplit * (2 + p.vdim);
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, w[z * (2 + p.vdim)]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = w[z * (2 + p.vdim)];
+    if (mz != -INFINITY) L += w[z * (2 + p.vdim) + 1] * __expf(mz - M);
+  }
+  float sig = p.out_scale;
+  if (p.gate) sig *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head]));
+  for (int col = threadIdx.x; col < p.vdim; col += blockDim.x) {
+    float o = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float mz = w[z * (2 + p.vdim)];
+      if (mz != -INFINITY) o += w[z * (2 + p.vdim) + 2 + col] * __expf(mz - M);
+    }
     p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(o * sig / L);
   }
 }
@@ -350,8 +451,8 @@ bool dba_decode_supported(int heads, int kv_heads, int dim, int vdim) {
   return qh * (1 << chl) <= 64;
 }
 
-void dba_decode_launch(const DBAParams& p, int64_t num_tokens, hipStream_t st) {
-  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads);
+void dba_decode_launch(const DBAParams& p, int64_t num_tokens, int nsplit, hipStream_t st) {
+  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)nsplit);
   const int qh = p.heads / p.kv_heads, chl = decode_chl(p.dim, p.vdim);
 #define DEC(QH, CHL) hipLaunchKernelGGL((dba_decode_kernel<QH, CHL>), grid, dim3(256), 0, st, p)
 #define DEC_BY_CHL(QH)                          \
@@ -369,6 +470,18 @@ void dba_decode_launch(const DBAParams& p, int64_t num_tokens, hipStream_t st) {
   }
 #undef DEC_BY_CHL
 #undef DEC
+  if (nsplit > 1)
+    hipLaunchKernelGGL(dba_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3(64), 0, st, p, nsplit);
+}
+
+// Key splits of the decode kernel: enough workgroups to fill the chip, at least four 64-key tiles (one per wave) each.
+int dba_decode_splits(int64_t num_tokens, int kv_heads, int max_kv_len, int64_t ws_floats, int heads, int vdim) {
+  const int tiles = (max_kv_len + 63) / 64;
+  int64_t n = (1024 + num_tokens * kv_heads - 1) / (num_tokens * kv_heads);
+  if (n > tiles / 4) n = tiles / 4;
+  if (n > 8) n = 8;
+  while (n > 1 && num_tokens * heads * n * (2 + vdim) > ws_floats) --n;
+  return n < 1 ? 1 : (int)n;
 }
 
 }  // namespace aphro

@@ -27,6 +27,24 @@ __device__ __forceinline__ float wg_sum(float v, float* red) {
   return t;
 }
 
+// Sums over groups of 2^LOG adjacent lanes with DPP moves (no LDS round trip): quad permutes for 2 and 4, the half-row and
+// row mirrors for 8 and 16 (after the quad steps every lane of a quad holds the quad's total, so the mirror partner brings
+// in the other half); every lane of a group ends with the group's total.  Wider groups finish with ds_bpermute shuffles.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LOG>
+__device__ __forceinline__ float group_sum(float v) {
+  if (LOG >= 1) v += dpp_f<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+  if (LOG >= 2) v += dpp_f<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+  if (LOG >= 3) v += dpp_f<0x141>(v);      // row_half_mirror
+  if (LOG >= 4) v += dpp_f<0x140>(v);      // row_mirror
+  if (LOG >= 5) v += __shfl_xor(v, 16, 64);
+  if (LOG >= 6) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + __expf(-z)); }
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + __expf(-z)); }
 __device__ __forceinline__ float gelu_tanh_f(float z) {

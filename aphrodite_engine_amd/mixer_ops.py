@@ -148,11 +148,13 @@ def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[t
                             v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                             ctx_len: torch.Tensor, seq_of_token: torch.Tensor, q_len_range, heads: int, scale: float,
                             bias_lut: Optional[torch.Tensor], temp_coef: float = 0.0, temp_every: int = 1,
-                            out_scale: float = 1.0) -> None:
+                            out_scale: float = 1.0, max_kv_len: int = 0) -> None:
     """Causal attention of a batch of segments over the paged cache, written into ``out`` [T, heads * e] (dense rows, any
     row stride).  q [T, heads * d]; gate [T, heads] raw (sigmoid inside) or None; bias_lut fp32 [heads, L] indexed by
     min(distance, L - 1) or None.  ``q_len_range``: (shortest, longest) segment of the batch, known on the host -- it
-    chooses between the matrix-core kernel for prompt portions and the shared-key kernel for single tokens."""
+    chooses between the matrix-core kernel for prompt portions and the shared-key kernel for single tokens.
+    ``max_kv_len``: the longest ctx_len + q_len of the batch (host); given, long key ranges of decoded rows are split over
+    several workgroups through a scratch tensor."""
     _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, q_len, ctx_len, seq_of_token, bias_lut)
     lo, hi = int(q_len_range[0]), int(q_len_range[1])
     _need(0 < lo <= hi, "distance_bias_attention: q_len_range (shortest, longest)")
@@ -178,16 +180,20 @@ def distance_bias_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[t
         _need(bias_lut.dtype == torch.float32 and bias_lut.dim() == 2 and bias_lut.shape[0] == heads and bias_lut.is_contiguous(),
               "distance_bias_attention: bias_lut fp32 [heads, L]")
         L = bias_lut.shape[1]
+    ws, ws_n = None, 0
+    if q.dtype == torch.bfloat16 and max_kv_len >= 512 and lo < 8:
+        ws_n = T * heads * 8 * (2 + e)
+        ws = torch.empty(ws_n, dtype=torch.float32, device=q.device)
     check(_lib.mixers_lib().aphro_distance_bias_attention(
         out.data_ptr(), _rows(out, heads * e, "out"), q.data_ptr(), _rows(q, heads * d, "q"), _p(gate), gs, k_cache.data_ptr(),
         v_cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(),
         ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, lo, hi, heads, G, d, e, float(scale), _p(bias_lut), L, float(temp_coef), int(temp_every),
-        float(out_scale), _dt(q), _stream()), "distance_bias_attention")
+        float(out_scale), int(max_kv_len), _p(ws), ws_n, _dt(q), _stream()), "distance_bias_attention")
 
 
 def memory_state_shapes(slots: int, heads: int, dim: int, vdim: int, mode: int):
     """Shapes of the fp32 state tensors of ``outer_memory_scan`` for a pool of ``slots`` requests."""
-    tiles = (vdim + 63) // 64
+    tiles = (vdim + 15) // 16
     s = (slots, heads, dim, vdim)
     return (s, ) if mode == MEMORY_DECAY else (s, (slots, heads, tiles, dim), (slots, heads, tiles))
 
@@ -195,9 +201,11 @@ def memory_state_shapes(slots: int, heads: int, dim: int, vdim: int, mode: int):
 def outer_memory_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state, slot_of_seq: torch.Tensor,
                       q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, heads: int, mode: int,
                       decay: Optional[torch.Tensor] = None, gate_i: Optional[torch.Tensor] = None,
-                      gate_f: Optional[torch.Tensor] = None, q_scale: float = 1.0, gate_cap: float = 1.0) -> torch.Tensor:
+                      gate_f: Optional[torch.Tensor] = None, q_scale: float = 1.0, gate_cap: float = 1.0,
+                      max_q_len: int = 1) -> torch.Tensor:
     """Scan every segment through its slot's state (updated in place); returns o fp32 [T, heads * vdim].  ``state`` is
-    the tuple of tensors shaped by ``memory_state_shapes``.  q, k [T, heads * d], v [T, heads * e]; gates [T, heads] raw."""
+    the tuple of tensors shaped by ``memory_state_shapes``.  q, k [T, heads * d], v [T, heads * e]; gates [T, heads] raw.
+    ``max_q_len`` (host: the batch's longest segment) picks the work split: wide for prompt portions, narrow for tokens."""
     _cuda(q, k, v, slot_of_seq, q_start, q_len, ctx_len, decay, gate_i, gate_f, *state)
     T = q.shape[0]
     S = q_start.numel()
@@ -223,5 +231,5 @@ def outer_memory_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state, 
         _rows(v, heads * e, "v"), _p(gate_i), _p(gate_f), gs, state[0].data_ptr(),
         state[1].data_ptr() if len(state) > 1 else None, state[2].data_ptr() if len(state) > 2 else None,
         slot_of_seq.data_ptr(), slots, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), S, T, heads, d, e, int(mode),
-        _p(decay), float(q_scale), float(gate_cap), _dt(q), _stream()), "outer_memory_scan")
+        _p(decay), float(q_scale), float(gate_cap), int(max_q_len), _dt(q), _stream()), "outer_memory_scan")
     return out

@@ -98,7 +98,8 @@ class DistanceBiasAttention(nn.Module):
         mops.paged_kv_write(k_cache, v_cache, k, v, batch.slot_mapping)
         mops.distance_bias_attention(out, q, gate, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len,
                                      batch.ctx_len, batch.seq_of_token, (min(batch.q_lens), max(batch.q_lens)), self.heads,
-                                     self.scale, self.bias_lut, self.temp_coef, self.temp_every, out_scale)
+                                     self.scale, self.bias_lut, self.temp_coef, self.temp_every, out_scale,
+                                     max_kv_len=max(c + n for c, n in zip(batch.ctx_lens, batch.q_lens)))
 
 
 class OuterProductMemory(nn.Module):
@@ -119,7 +120,8 @@ class OuterProductMemory(nn.Module):
 
     def forward(self, q, k, v, state, batch: StepBatch, gate_i=None, gate_f=None) -> torch.Tensor:
         return mops.outer_memory_scan(q, k, v, state, batch.state_slots, batch.q_start, batch.q_len, batch.ctx_len,
-                                      self.heads, self.mode, self.decay, gate_i, gate_f, self.q_scale, self.gate_cap)
+                                      self.heads, self.mode, self.decay, gate_i, gate_f, self.q_scale, self.gate_cap,
+                                      max_q_len=max(batch.q_lens))
 
 
 class GatedMLP(nn.Module):

@@ -68,14 +68,17 @@ int aphro_paged_kv_write(void* k_cache, void* v_cache, const void* k, int64_t k_
  * Query head h reads key/value head h / (heads / kv_heads).  q_len int32 [num_seqs] with its host-side minimum and
  * maximum choose the kernels: bf16 segments of 8 rows or more run on the matrix cores (dim, vdim in {32, 64, 96, 128}),
  * shorter ones on a kernel that reads each key once for all query heads of its kv head (dim, vdim multiples of 8, at most
- * 256, 1 / 2 / 4 / 8 query heads per kv head); every other case -- and fp32 -- runs the scalar fp32 kernel. */
+ * 256, 1 / 2 / 4 / 8 query heads per kv head); every other case -- and fp32 -- runs the scalar fp32 kernel.
+ * max_kv_len (host-side longest ctx_len + q_len) and an optional fp32 workspace let the shared-key kernel split long key
+ * ranges over up to 8 workgroups per row (num_tokens * heads * splits * (2 + vdim) floats; NULL: no split). */
 int aphro_distance_bias_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
                                   int64_t gate_stride, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                   int max_blocks, int64_t num_blocks, int block_size, const int32_t* q_start,
                                   const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token,
                                   int64_t num_tokens, int num_seqs, int min_q_len, int max_q_len, int heads, int kv_heads,
                                   int dim, int vdim, float scale, const float* bias_lut, int lut_len, float temp_coef,
-                                  int temp_every, float out_scale, int dtype, void* stream);
+                                  int temp_every, float out_scale, int max_kv_len, float* workspace,
+                                  int64_t workspace_floats, int dtype, void* stream);
 
 /* Gated outer-product memory, one state per (slot, head):  S <- a_t S + b_t k_t v_t^T,  o_t = S^T q_t  [/ normaliser].
  *   mode 0 (decay linear attention): q, k, v = silu(raw); a_t = decay[h], b_t = 1.
@@ -84,15 +87,16 @@ int aphro_distance_bias_attention(void* out, int64_t out_stride, const void* q, 
  *     o_t = S^T q_t / (max(|n . q_t|, exp(-m_t)) + 1e-6).  m, n and S start at zero.
  * q, k [T, heads * dim], v [T, heads * vdim], gates [T, heads] (row strides) of `dtype`; out fp32 [T, heads * vdim].
  * state_s fp32 [slots, heads, dim, vdim]; mode 1 only: state_n fp32 [slots, heads, tiles, dim] and state_m fp32
- * [slots, heads, tiles], tiles = ceil(vdim / 64) (every 64-column tile of the launch keeps its own copy of n and m, so no
- * workgroup reads what another one writes).  slot_of_seq int32 [num_seqs]; a segment with ctx_len == 0 starts from zero
+ * [slots, heads, tiles], tiles = ceil(vdim / 16) (every 16 value columns keep their own copy of n and m, so no workgroup
+ * reads what another one writes, whichever of the two work splits -- chosen by max_q_len, the host-side longest segment --
+ * a launch uses).  slot_of_seq int32 [num_seqs]; a segment with ctx_len == 0 starts from zero
  * without reading its slot. */
 int aphro_outer_memory_scan(float* out, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                             int64_t v_stride, const void* gate_i, const void* gate_f, int64_t gate_stride, float* state_s,
                             float* state_n, float* state_m, const int32_t* slot_of_seq, int num_slots,
                             const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len, int num_seqs,
                             int64_t num_tokens, int heads, int dim, int vdim, int mode, const float* decay, float q_scale,
-                            float gate_cap, int dtype, void* stream);
+                            float gate_cap, int max_q_len, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -126,7 +126,7 @@ def run_attention(mops, pg, qs, ctx, H, scale, lut, coef, every, dtype, gate=Non
     out = torch.full((q.shape[0], H * e + 3), 7.0, dtype=dtype, device=DEV)
     mops.distance_bias_attention(out[:, :H * e], q, None if gate is None else dev(gate, dtype), pg.kc, pg.vc, bt,
                                  i32(starts), i32(lens), i32(ctx), i32(seq_of), (min(lens), max(lens)), H, scale, lut, coef, every,
-                                 out_scale)
+                                 out_scale, max_kv_len=max(a + b for a, b in zip(ctx, lens)))
     assert float((out[:, H * e:] - 7.0).abs().sum()) == 0
     return out[:, :H * e].float().cpu().numpy().reshape(-1, H, e)
 
@@ -171,6 +171,25 @@ def test_attention_prompt_portion_and_decode(mops, dtype, shape):
     np.testing.assert_allclose(got, np.concatenate([want[2][36:37], want[0][37:99]]), rtol=tol, atol=tol)
     got = run_attention(mops, pg, [q[0][148:150]], [148], H, scale, lut, coef, every, dtype, seqs=[0])
     np.testing.assert_allclose(got, want[0][148:150], rtol=tol, atol=tol)
+
+
+def test_decoded_rows_over_long_contexts_split_their_keys(mops):
+    """bfloat16 rows with a long context are split over several workgroups and merged; short and long contexts, a
+    three-token portion and a prompt portion share the batch."""
+    H, G, d, e = 8, 2, 64, 128
+    rng = np.random.default_rng(11)
+    lens = [1500, 700, 40, 900]
+    dt = torch.bfloat16
+    q = [rounded(rng.standard_normal((n, H, d)), dt) for n in lens]
+    k = [rounded(rng.standard_normal((n, G, d)), dt) for n in lens]
+    v = [rounded(rng.standard_normal((n, G, e)), dt) for n in lens]
+    rel = rng.standard_normal((10, H)).astype(np.float32)
+    want = [O.biased_softmax_attention(q[s], k[s], v[s], rel.astype(np.float64), d ** -0.5, 300, 0.3, 128) for s in range(4)]
+    pg, lut = Paged(mops, k, v, dt), make_lut(rel, 300)
+    got = run_attention(mops, pg, [q[3][880:900], q[0][1499:], q[1][697:], q[2][39:]], [880, 1499, 697, 39], H, d ** -0.5, lut, 0.3,
+                        128, dt, seqs=[3, 0, 1, 2])
+    w = np.concatenate([want[3][880:900], want[0][1499:], want[1][697:], want[2][39:]])
+    np.testing.assert_allclose(got, w, rtol=2.5e-2, atol=2.5e-2)
 
 
 @pytest.mark.parametrize("decoded", [False, True])
@@ -267,7 +286,7 @@ def scan_in_steps(mops, mode, q, k, v, cuts, dtype, decay=None, gi=None, gf=None
         else:
             kw = dict(decay=torch.tensor(decay, dtype=torch.float32, device=DEV))
         o = mops.outer_memory_scan(cat(q, 5), cat(k), cat(v, 1), state, i32([slot_of[s] for s in live]), i32(starts), i32(lens),
-                                   i32([a for a, _ in seg]), H, mode, **kw).cpu().numpy()
+                                   i32([a for a, _ in seg]), H, mode, max_q_len=max(lens), **kw).cpu().numpy()
         for s, (a, b), st in zip(live, seg, starts):
             outs[s][a:b] = o[st:st + b - a]
     return outs
@@ -285,7 +304,7 @@ def test_decay_memory_in_steps(mops, dtype, shape):
     decay = [0.999, 0.6, 0.9, 0.3, 0.97][:H]
     want = [O.decay_linear_attention(O.silu(q[s]), O.silu(k[s]), O.silu(v[s]), np.array(decay)).reshape(lens[s], -1)
             for s in range(3)]
-    for cuts in ([[], [], []], [[16, 17, 19, 48, 64], [], [2, 4, 31]], [list(range(1, 70)), [], [32]]):
+    for cuts in ([[], [], []], [[16, 17, 19, 48, 64], [], [2, 4, 31]], [list(range(1, 70)), [], [32]], [[40], [], [32]], [[3, 69], [], []]):
         got = scan_in_steps(mops, mops.MEMORY_DECAY, q, k, v, cuts, dtype, decay=decay)
         for s in range(3):
             np.testing.assert_allclose(got[s], want[s], rtol=3e-5, atol=3e-5 * np.abs(want[s]).max())
@@ -309,7 +328,7 @@ def test_mlstm_memory_in_steps(mops, dtype, shape):
         i_log = cap * np.tanh(gi[s] / cap)
         f_log = O.log_sigmoid(cap * np.tanh(gf[s] / cap))
         want.append(O.mlstm_memory(q[s] * d ** -0.5, k[s], v[s], i_log, f_log).reshape(lens[s], -1))
-    for cuts in ([[], [], []], [[16, 17, 19, 48, 64], [], [2, 4, 31]], [list(range(1, 70)), [], [32]]):
+    for cuts in ([[], [], []], [[16, 17, 19, 48, 64], [], [2, 4, 31]], [list(range(1, 70)), [], [32]], [[40], [], [32]], [[3, 69], [], []]):
         got = scan_in_steps(mops, mops.MEMORY_MLSTM, q, k, v, cuts, dtype, gi=gi, gf=gf, q_scale=d ** -0.5, cap=cap)
         for s in range(3):
             np.testing.assert_allclose(got[s], want[s], rtol=1e-4, atol=1e-4 * np.abs(want[s]).max())
