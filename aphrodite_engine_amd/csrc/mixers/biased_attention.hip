@@ -169,6 +169,7 @@ struct DBAParams {
   float scale, temp_coef, out_scale;
   float* ws;
   int bs_shift;
+  int max_tiles;
 };
 bool dba_prefill_supported(int dim, int vdim);
 bool dba_decode_supported(int heads, int kv_heads, int dim, int vdim);
@@ -229,6 +230,7 @@ extern "C" int aphro_distance_bias_attention(void* out, int64_t out_stride, cons
     p.max_blocks = max_blocks; p.block_size = block_size; p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim;
     p.lut_len = lut_len; p.temp_every = temp_every; p.scale = scale; p.temp_coef = temp_coef; p.out_scale = out_scale;
     p.ws = workspace;
+    p.max_tiles = 0;
     p.bs_shift = -1;
     for (int sft = 0; sft < 20; ++sft)
       if ((1 << sft) == block_size) p.bs_shift = sft;

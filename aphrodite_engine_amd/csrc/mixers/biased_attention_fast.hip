@@ -37,6 +37,7 @@ struct DBAParams {          // (declared alike in biased_attention.hip, which fi
   float scale, temp_coef, out_scale;
   float* ws;          // decode split partials [T, heads, nsplit, 2 + vdim]
   int bs_shift;       // log2(block_size), or -1 when it is no power of two
+  int max_tiles;      // prompt kernel: 64-row tiles of the longest segment
 };
 
 // row of key `key` in the token-major cache ([block, offset] -> block * block_size + offset), following the block table
@@ -122,41 +123,69 @@ __device__ __forceinline__ void pf_store(const PFStage<DK, DV>& st, uint16_t* k_
   }
 }
 
-template <int DK, int DV>
+// QT query heads of one kv head share a workgroup: the K and V fragments read from LDS feed QT products each, and the
+// tile's trip from the cache to LDS is paid once for them.
+template <int DK, int DV, int QT>
 __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
   constexpr int NCHK = DK / 8, NKS = DK / 32, NDT = DV / 16, NH = PF_BN / 16, NPK = PF_BN / 32;
   constexpr int SWZ = (NCHK & -NCHK) - 1;
   constexpr int NWIN = PF_BM + PF_BN - 1;
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[PF_BN * DK];
   __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DV * PF_VT];
-  __shared__ float bias_win[NWIN + 1];
+  __shared__ float bias_win[QT][NWIN + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
-  const int head = blockIdx.y, seq = blockIdx.z;
+  const int seq = blockIdx.y;
   const int len = p.q_len[seq];
   if (len < p.min_len) return;
   const int ntiles = (len + PF_BM - 1) / PF_BM;
-  const int tile = ntiles - 1 - (int)blockIdx.x;           // the longest key ranges first
-  if (tile < 0) return;
+  // Workgroups go to the 8 XCDs round-robin by their linear index, and each XCD has its own L2: the (tile, head unit) pairs
+  // are numbered so that every query head of one kv head -- the workgroups that read the same keys and values -- lands on
+  // the same XCD (or the same few, when there are fewer kv heads than XCDs).  Within an XCD: longest key ranges first.
+  int unit, rank;                                           // head unit: QT consecutive query heads
+  {
+    constexpr int NX = 8;
+    const int G = p.kv_heads, QU = p.heads / p.kv_heads / QT, x = blockIdx.x % NX, j = blockIdx.x / NX;
+    if (G % NX == 0) {
+      const int ux = (G / NX) * QU, ul = j % ux;            // units served by this XCD, this workgroup's among them
+      rank = j / ux;
+      unit = ((ul / QU) * NX + x) * QU + ul % QU;
+    } else if (NX % G == 0) {
+      const int share = NX / G, pair = j * share + x / G;   // XCDs per kv head; (tile, unit) pair of that kv head
+      rank = pair / QU;
+      unit = (x % G) * QU + pair % QU;
+    } else {
+      rank = blockIdx.x / (p.heads / QT);
+      unit = blockIdx.x % (p.heads / QT);
+    }
+  }
+  const int tile = ntiles - 1 - rank;
+  if (tile < 0 || rank >= p.max_tiles) return;
+  const int head0 = unit * QT;
   const int ctx = p.ctx_len[seq], s0 = p.q_start[seq];
-  const int kvh = head / (p.heads / p.kv_heads);
+  const int kvh = head0 / (p.heads / p.kv_heads);
   const int q0 = tile * PF_BM;
   const int qrow = q0 + 16 * wave + c;
   const bool qvalid = qrow < len;
   const int qpos = ctx + qrow;
   constexpr float LOG2E = 1.4426950408889634f;
   const float qs = p.scale * dba_temp(p, qpos) * LOG2E;     // scores in units of ln 2: the exponentials are exp2
-  u32x4 qf[NKS];
-  {
-    const uint16_t* qp = p.q + (int64_t)(s0 + min(qrow, len - 1)) * p.q_stride + head * DK;
+  u32x4 qf[QT][NKS];
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const u32x4*>(qp + 32 * ks + 8 * g);
+  for (int t = 0; t < QT; ++t) {
+    const uint16_t* qp = p.q + (int64_t)(s0 + min(qrow, len - 1)) * p.q_stride + (head0 + t) * DK;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qf[t][ks] = *reinterpret_cast<const u32x4*>(qp + 32 * ks + 8 * g);
   }
-  f32x4 o[NDT];
+  f32x4 o[QT][NDT];
+  float m_run[QT], l_run[QT];
 #pragma unroll
-  for (int i = 0; i < NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -1e30f, l_run = 0.f;
+  for (int t = 0; t < QT; ++t) {
+    m_run[t] = -1e30f;
+    l_run[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) o[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
-  const float* lut = p.bias_lut ? p.bias_lut + (int64_t)head * p.lut_len : nullptr;
   const int nk = ctx + min(len, q0 + PF_BM);               // keys the tile's last row sees
 
   PFStage<DK, DV> st;
@@ -165,83 +194,103 @@ __global__ __launch_bounds__(256) void dba_prefill_kernel(DBAParams p) {
     __syncthreads();                                        // the previous tile is consumed
     pf_store<DK, DV>(st, k_lds, vt_lds);
     const int dmin = ctx + q0 - t0 - (PF_BN - 1);           // distance of (first row, last key of the tile)
-    if (threadIdx.x < NWIN) {
-      float b = 0.f;
-      if (lut) {
-        const int dist = dmin + (int)threadIdx.x;
-        b = lut[dist < 0 ? 0 : (dist < p.lut_len ? dist : p.lut_len - 1)] * LOG2E;
+    if (threadIdx.x < QT * 128) {
+      const int t = threadIdx.x >> 7, x = threadIdx.x & 127;
+      if (x < NWIN) {
+        float b = 0.f;
+        if (p.bias_lut) {
+          const int dist = dmin + x;
+          b = p.bias_lut[(int64_t)(head0 + t) * p.lut_len + (dist < 0 ? 0 : (dist < p.lut_len ? dist : p.lut_len - 1))] * LOG2E;
+        }
+        bias_win[t][x] = b;
       }
-      bias_win[threadIdx.x] = b;
     }
     __syncthreads();
     if (t0 + PF_BN < nk) pf_load<DK, DV>(st, p, bt, kvh, t0 + PF_BN, nk);      // in flight during this tile's products
     if (t0 > ctx + q0 + 16 * wave + 15) continue;           // every key of the tile is ahead of the wave's rows
-    f32x4 s[NH];
+    f32x4 s[QT][NH];
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
-      s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < QT; ++t) s[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
       const int tok = 16 * h + c;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const int ch = (4 * ks + g) ^ (tok & SWZ);
         const u32x4 kf = *reinterpret_cast<const u32x4*>(&k_lds[tok * DK + 8 * ch]);
-        s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < QT; ++t)
+          s[t][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[t][ks]),
+                                                            s[t][h], 0, 0, 0);
       }
     }
-    float pv[NH][4];
-    float mx = -1e30f;
-    const float* bw = &bias_win[qpos - t0 - dmin - 4 * g];  // bias of (this row, key t0 + 4 g); keys count downwards
     const bool diag = t0 + PF_BN - 1 > ctx + q0 + 16 * wave; // some key of the tile is ahead of some row of the wave
+    u32x4 pf[QT][NPK];
 #pragma unroll
-    for (int h = 0; h < NH; ++h)
+    for (int t = 0; t < QT; ++t) {
+      float pv[NH][4];
+      float mx = -1e30f;
+      const float* bw = &bias_win[t][qpos - t0 - dmin - 4 * g];    // bias of (this row, key t0 + 4 g); keys count downwards
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float xv = s[h][r] * qs + bw[-(16 * h + r)];
-        if (diag) xv = t0 + 16 * h + 4 * g + r <= qpos ? xv : -1e30f;
-        pv[h][r] = xv;
-        mx = fmaxf(mx, xv);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);                   // finite for every row that is kept: key 0 is visible
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
-    float lsum = 0.f;
+      for (int h = 0; h < NH; ++h)
 #pragma unroll
-    for (int h = 0; h < NH; ++h)
+        for (int r = 0; r < 4; ++r) {
+          float xv = s[t][h][r] * qs + bw[-(16 * h + r)];
+          if (diag) xv = t0 + 16 * h + 4 * g + r <= qpos ? xv : -1e30f;
+          pv[h][r] = xv;
+          mx = fmaxf(mx, xv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[t], mx);              // finite for every row that is kept: key 0 is visible
+      const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_new);
+      m_run[t] = m_new;
+      float lsum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float e = __builtin_amdgcn_exp2f(pv[h][r] - m_new);           // a masked score is 1e30 below: exactly 0
-        pv[h][r] = e;
-        lsum += e;
-      }
-    l_run = l_run * alpha + lsum;
+      for (int h = 0; h < NH; ++h)
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) o[dt] *= alpha;
+        for (int r = 0; r < 4; ++r) {
+          const float e = __builtin_amdgcn_exp2f(pv[h][r] - m_new);    // a masked score is 1e30 below: exactly 0
+          pv[h][r] = e;
+          lsum += e;
+        }
+      l_run[t] = l_run[t] * alpha + lsum;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) o[t][dt] *= alpha;
+#pragma unroll
+      for (int pk = 0; pk < NPK; ++pk)
+        pf[t][pk] = u32x4{pack2_16<true>(pv[2 * pk][0], pv[2 * pk][1]), pack2_16<true>(pv[2 * pk][2], pv[2 * pk][3]),
+                          pack2_16<true>(pv[2 * pk + 1][0], pv[2 * pk + 1][1]), pack2_16<true>(pv[2 * pk + 1][2], pv[2 * pk + 1][3])};
+    }
 #pragma unroll
     for (int pk = 0; pk < NPK; ++pk) {
-      const u32x4 pf = {pack2_16<true>(pv[2 * pk][0], pv[2 * pk][1]), pack2_16<true>(pv[2 * pk][2], pv[2 * pk][3]),
-                        pack2_16<true>(pv[2 * pk + 1][0], pv[2 * pk + 1][1]), pack2_16<true>(pv[2 * pk + 1][2], pv[2 * pk + 1][3])};
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
         const uint16_t* vr = &vt_lds[(16 * dt + c) * PF_VT + 32 * pk + 4 * g];
         const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
         const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < QT; ++t)
+          o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[t][pk]),
+                                                             o[t][dt], 0, 0, 0);
       }
     }
   }
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  if (!qvalid) return;
-  float f = (l_run > 0.f ? 1.f / l_run : 0.f) * p.out_scale;
-  if (p.gate) f *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)(s0 + qrow) * p.gate_stride + head]));
-  uint16_t* op = p.out + (int64_t)(s0 + qrow) * p.out_stride + head * DV;
+  if (!qvalid) return;                                      // (after the last shuffle-free point: the sums below are per lane group)
 #pragma unroll
-  for (int dt = 0; dt < NDT; ++dt) {
+  for (int t = 0; t < QT; ++t) {
+    float l = l_run[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    float f = (l > 0.f ? 1.f / l : 0.f) * p.out_scale;
+    if (p.gate) f *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)(s0 + qrow) * p.gate_stride + head0 + t]));
+    uint16_t* op = p.out + (int64_t)(s0 + qrow) * p.out_stride + (head0 + t) * DV;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) op[16 * dt + 4 * g + r] = BFloat::from_f32(o[dt][r] * f);
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) op[16 * dt + 4 * g + r] = BFloat::from_f32(o[t][dt][r] * f);
+    }
   }
 }
 
@@ -410,15 +459,14 @@ __global__ void dba_merge_kernel(DBAParams p, int nsplit) {
   }
 }
 
-template <int DK>
-static bool launch_prefill_dv(const DBAParams& p, dim3 grid, hipStream_t st) {
+template <int DK, int QT>
+static void launch_prefill_dv(const DBAParams& p, dim3 grid, hipStream_t st) {
   switch (p.vdim) {
-    case 32: hipLaunchKernelGGL((dba_prefill_kernel<DK, 32>), grid, dim3(256), 0, st, p); return true;
-    case 64: hipLaunchKernelGGL((dba_prefill_kernel<DK, 64>), grid, dim3(256), 0, st, p); return true;
-    case 96: hipLaunchKernelGGL((dba_prefill_kernel<DK, 96>), grid, dim3(256), 0, st, p); return true;
-    case 128: hipLaunchKernelGGL((dba_prefill_kernel<DK, 128>), grid, dim3(256), 0, st, p); return true;
+    case 32: hipLaunchKernelGGL((dba_prefill_kernel<DK, 32, QT>), grid, dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((dba_prefill_kernel<DK, 64, QT>), grid, dim3(256), 0, st, p); break;
+    case 96: hipLaunchKernelGGL((dba_prefill_kernel<DK, 96, QT>), grid, dim3(256), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((dba_prefill_kernel<DK, 128, QT>), grid, dim3(256), 0, st, p); break;
   }
-  return false;
 }
 
 bool dba_prefill_supported(int dim, int vdim) {
@@ -426,14 +474,24 @@ bool dba_prefill_supported(int dim, int vdim) {
   return ok(dim) && ok(vdim);
 }
 
-void dba_prefill_launch(const DBAParams& p, int max_q_len, int num_seqs, hipStream_t st) {
-  const dim3 grid((unsigned)((max_q_len + PF_BM - 1) / PF_BM), (unsigned)p.heads, (unsigned)num_seqs);
+template <int QT>
+static void launch_prefill_dk(const DBAParams& p, dim3 grid, hipStream_t st) {
   switch (p.dim) {
-    case 32: launch_prefill_dv<32>(p, grid, st); break;
-    case 64: launch_prefill_dv<64>(p, grid, st); break;
-    case 96: launch_prefill_dv<96>(p, grid, st); break;
-    case 128: launch_prefill_dv<128>(p, grid, st); break;
+    case 32: launch_prefill_dv<32, QT>(p, grid, st); break;
+    case 64: launch_prefill_dv<64, QT>(p, grid, st); break;
+    case 96: launch_prefill_dv<96, QT>(p, grid, st); break;
+    case 128: launch_prefill_dv<128, QT>(p, grid, st); break;
   }
+}
+
+void dba_prefill_launch(const DBAParams& p0, int max_q_len, int num_seqs, hipStream_t st) {
+  DBAParams p = p0;
+  p.max_tiles = (max_q_len + PF_BM - 1) / PF_BM;
+  const int qt = (p.heads / p.kv_heads) % 2 == 0 ? 2 : 1;   // two query heads of a kv head per workgroup where they pair up
+  const int per_seq = (p.max_tiles * (p.heads / qt) + 7) / 8 * 8;      // a multiple of the XCD count: the numbering repeats per segment
+  const dim3 grid((unsigned)per_seq, (unsigned)num_seqs);
+  if (qt == 2) launch_prefill_dk<2>(p, grid, st);
+  else launch_prefill_dk<1>(p, grid, st);
 }
 
 // lanes per key row: the smallest power of two that covers both row lengths in 16-byte pieces

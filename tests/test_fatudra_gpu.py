@@ -144,6 +144,8 @@ ATT_SHAPES = [  # H, G, d, e, rows, far, coef, every
     (3, 3, 20, 72, 9, 33.5, 2.0, 7),          # no grouping, odd table, sizes that force the scalar loads
     (8, 2, 64, 128, 16, 100, 0.0, 1),         # vector loads, two output columns per lane, no temperature
     (2, 1, 96, 200, 6, 20, 0.25, 5),
+    (3, 3, 32, 64, 7, 45, 0.4, 11),           # one query head per kv head: the unpaired matrix-core form
+    (6, 2, 64, 32, 8, 60, 0.3, 9),            # three query heads per kv head: no shared-key form, long segments only on the matrix cores
 ]
 
 
