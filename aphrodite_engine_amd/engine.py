@@ -215,6 +215,10 @@ class LLMEngine:
         and keeps its pages and slot until ``release``.  Returns fp32 logits of the wanted places, in order."""
         segments, want = [], []
         for rid, toks, w in entries:
+            if len(toks) == 0:
+                if len(w):
+                    raise ValueError(f"request {rid}: logits wanted of an entry without tokens")
+                continue
             r = self.requests.get(rid)
             if r is None:
                 r = Request(rid, [], 0)
@@ -227,6 +231,8 @@ class LLMEngine:
             r.num_prompt = len(r.tokens)
             segments.append((r, toks))
             want.append(list(w))
+        if not segments:
+            return torch.empty(0, self.runner.model.vocab_size, dtype=torch.float32, device=self.runner.device)
         # prompt portions first, decoded tokens last (the order attention metadata assumes); answers keep the caller's order
         order = sorted(range(len(segments)), key=lambda i: len(segments[i][1]) == 1 and segments[i][0].num_computed > 0)
         logits = self._run([segments[i] for i in order], [want[i] for i in order])
