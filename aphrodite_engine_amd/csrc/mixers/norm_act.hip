@@ -88,6 +88,116 @@ __global__ void residual_layer_norm_kernel(float* __restrict__ residual, const t
     o[i] = T::from_f32((row[i] - mean) * rstd * T::to_f32(pre_w[i]) + T::to_f32(pre_b[i]));
 }
 
+// ---- the same two kernels for rows that are a multiple of 8 elements and 16-byte aligned: every thread owns 8 consecutive
+// elements in registers (no LDS row), all of a row's inputs are requested before the first reduction.
+template <typename T>
+__device__ __forceinline__ void load8(const typename T::storage* p, float* o) {
+  if constexpr (sizeof(typename T::storage) == 2) {
+    const u16x8 v = *reinterpret_cast<const u16x8*>(p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = T::to_f32(v[j]);
+  } else {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[j] = a[j];
+      o[4 + j] = b[j];
+    }
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store8(typename T::storage* p, const float* v) {
+  if constexpr (sizeof(typename T::storage) == 2) {
+    u16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = T::from_f32(v[j]);
+    *reinterpret_cast<u16x8*>(p) = r;
+  } else {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4*>(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+  }
+}
+
+__device__ __forceinline__ void stats8(const float* x, bool act, int width, float eps, float* red, float& mean, float& rstd) {
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s += act ? x[j] : 0.f;
+  mean = wg_sum(s, red) / (float)width;
+  float v = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float d = act ? x[j] - mean : 0.f;
+    v += d * d;
+  }
+  rstd = 1.0f / sqrtf(wg_sum(v, red) / (float)width + eps);
+}
+
+template <typename T>
+__global__ void residual_layer_norm_vec8_kernel(float* __restrict__ residual, const typename T::storage* __restrict__ y,
+                                                int64_t y_stride, const float* __restrict__ y_bias,
+                                                const typename T::storage* __restrict__ post_w,
+                                                const typename T::storage* __restrict__ post_b,
+                                                const typename T::storage* __restrict__ add_vec,
+                                                const typename T::storage* __restrict__ pre_w,
+                                                const typename T::storage* __restrict__ pre_b,
+                                                typename T::storage* __restrict__ out, int width, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int i0 = threadIdx.x * 8;
+  const bool act = i0 < width;
+  const int ia = act ? i0 : 0;
+  float* r = residual + t * (int64_t)width;
+  float x[8], rv[8], w[8], b[8], av[8], qw[8], qb[8];
+  load8<Float>(r + ia, rv);
+  if (y) {
+    load8<T>(y + t * y_stride + ia, x);
+    load8<T>(post_w + ia, w);
+    load8<T>(post_b + ia, b);
+    if (y_bias) {
+      float yb[8];
+      load8<Float>(y_bias + ia, yb);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += yb[j];
+    }
+  }
+  if (add_vec) load8<T>(add_vec + ia, av);
+  if (out) {
+    load8<T>(pre_w + ia, qw);
+    load8<T>(pre_b + ia, qb);
+  }
+  if (y) {
+    float mean, rstd;
+    stats8(x, act, width, eps, red, mean, rstd);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rv[j] += (x[j] - mean) * rstd * w[j] + b[j];
+  }
+  if (add_vec) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rv[j] += av[j];
+  }
+  if ((y || add_vec) && act) store8<Float>(r + i0, rv);
+  if (out == nullptr) return;
+  float mean, rstd;
+  stats8(rv, act, width, eps, red, mean, rstd);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = (rv[j] - mean) * rstd * qw[j] + qb[j];
+  if (act) store8<T>(out + t * (int64_t)width + i0, x);
+}
+
+template <typename T, int ACT>
+__global__ void act_and_mul_vec8_kernel(typename T::storage* __restrict__ out, const typename T::storage* __restrict__ in,
+                                        int64_t in_stride, int d) {
+  const int64_t t = blockIdx.y;
+  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i0 >= d) return;
+  float g[8], u[8];
+  load8<T>(in + t * in_stride + i0, g);
+  load8<T>(in + t * in_stride + d + i0, u);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g[j] = (ACT == 0 ? silu_f(g[j]) : gelu_tanh_f(g[j])) * u[j];
+  store8<T>(out + t * (int64_t)d + i0, g);
+}
+
 template <typename T, int ACT>
 __global__ void act_and_mul_kernel(typename T::storage* __restrict__ out, const typename T::storage* __restrict__ in,
                                    int64_t in_stride, int d) {
@@ -149,6 +259,20 @@ extern "C" int aphro_residual_layer_norm(float* residual, const void* y, int64_t
   APHRO_CHECK(!y || (post_w && post_b && y_stride >= width), "residual_layer_norm: y needs post_w, post_b and a row stride >= width");
   APHRO_CHECK(!out || (pre_w && pre_b), "residual_layer_norm: out needs pre_w and pre_b");
   APHRO_CHECK(y || add_vec || out, "residual_layer_norm: nothing to do");
+  const auto al16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+  const bool vec = (width & 7) == 0 && width <= 8192 && (y_stride & 7) == 0 && al16(residual) && al16(y) && al16(y_bias) &&
+                   al16(post_w) && al16(post_b) && al16(add_vec) && al16(pre_w) && al16(pre_b) && al16(out);
+  if (vec) {
+    const int threads = ((width / 8) + 63) / 64 * 64;
+    MIX_DISPATCH_DTYPE(dtype, {
+      typedef typename T::storage S;
+      hipLaunchKernelGGL((residual_layer_norm_vec8_kernel<T>), dim3((unsigned)num_tokens), dim3(threads), 0, (hipStream_t)stream,
+                         residual, (const S*)y, y_stride, y_bias, (const S*)post_w, (const S*)post_b, (const S*)add_vec,
+                         (const S*)pre_w, (const S*)pre_b, (S*)out, width, eps);
+    });
+    APHRO_LAUNCH_CHECK();
+    return APHRO_OK;
+  }
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
     hipLaunchKernelGGL((residual_layer_norm_kernel<T>), dim3((unsigned)num_tokens), dim3(block_for(width)),
@@ -164,6 +288,19 @@ extern "C" int aphro_act_and_mul(void* out, const void* in, int64_t in_stride, i
                                  void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && in && d > 0 && in_stride >= 2 * (int64_t)d && (act == 0 || act == 1), "act_and_mul: bad arguments");
+  if ((d & 7) == 0 && (in_stride & 7) == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 && num_tokens <= 65535) {
+    const int per_row = d / 8, threads = per_row >= 256 ? 256 : (per_row + 63) / 64 * 64;
+    const dim3 grid((unsigned)((per_row + threads - 1) / threads), (unsigned)num_tokens);
+    MIX_DISPATCH_DTYPE(dtype, {
+      typedef typename T::storage S;
+      if (act == 0)
+        hipLaunchKernelGGL((act_and_mul_vec8_kernel<T, 0>), grid, dim3(threads), 0, (hipStream_t)stream, (S*)out, (const S*)in, in_stride, d);
+      else
+        hipLaunchKernelGGL((act_and_mul_vec8_kernel<T, 1>), grid, dim3(threads), 0, (hipStream_t)stream, (S*)out, (const S*)in, in_stride, d);
+    });
+    APHRO_LAUNCH_CHECK();
+    return APHRO_OK;
+  }
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
     if (act == 0)

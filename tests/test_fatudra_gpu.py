@@ -41,7 +41,7 @@ def rounded(a, dtype):
 # kernels alone
 # ---------------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [72, 200, 1032])
+@pytest.mark.parametrize("width", [72, 75, 200, 1032])      # 75: rows that cannot be read 16 bytes at a time
 def test_residual_layer_norm_all_steps(mops, dtype, width):
     rng = np.random.default_rng(width)
     T, eps = 5, 1e-5
