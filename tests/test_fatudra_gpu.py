@@ -489,3 +489,50 @@ def test_greedy_generation_through_the_scheduler(mops, tmp_path):
             seq.append(int(np.argmax(O.forward(cfg, W, seq)[-1])))
         assert out == seq[len(p):]
     assert eng.pages.num_free == eng.pages.total and eng.slots.num_free == 2 and not eng.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_command_on_an_unseen_shape(mops, tmp_path, dtype):
+    """bin/trace_run end to end: a checkpoint of sizes no other test uses (head sizes off the matrix-core list, one memory
+    head, a loop in the middle run three times), a schedule with portions beside single tokens and a request that ends,
+    the logits files against the restatement."""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg = U.make_config([U.mlstm_layer(heads=1, dim=24, vdim=56), U.parallel_layer(heads=5, kv_heads=5, dim=48, vdim=80, rheads=1,
+                                                                                   rdim=24, rvdim=40, bias_max=19, every=3),
+                         U.parallel_layer(heads=4, kv_heads=1, dim=64, vdim=32, rheads=2, rdim=32, rvdim=16, mlp=False)],
+                        vocab=300, width=96, loop=(1, 2, 3), embed_scale=3.0)
+    W = U.make_weights(cfg, seed=21, bias_rows=9)
+    model_dir = U.write_checkpoint(str(tmp_path / "m"), cfg, W)
+    ps = prompts(cfg, [75, 20, 2], seed=9)
+    want = [O.forward(cfg, W, p) for p in ps]
+    plan = [[(0, 40), (1, 2)], [(0, 1), (1, 1), (2, 2)], [(0, 20), (1, 17)], [(0, 14)]]
+    at, lines, rows = [0, 0, 0], [], []
+    for n, step in enumerate(plan):
+        entries, end = [], []
+        for i, k in step:
+            w = list(range(0, k, 2)) if k > 2 else list(range(k))
+            entries.append({"id": "q%d" % i, "tokens": ps[i][at[i]:at[i] + k], "want": w})
+            rows.append([(i, at[i] + x) for x in w])
+            at[i] += k
+            if at[i] == len(ps[i]):
+                end.append("q%d" % i)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype, "--out", str(out),
+                        "--max-tokens", "128"], input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == ["done %d" % n for n in range(len(plan))]
+    got, exp, k = [], [], 0
+    for n, step in enumerate(plan):
+        g = np.fromfile(str(out / ("%d.f32" % n)), dtype="<f4").reshape(-1, cfg["vocab"])
+        need = sum(len(rows[k + j]) for j in range(len(step)))
+        assert g.shape[0] == need
+        got.append(g)
+        for j in range(len(step)):
+            exp += [want[i][pos] for i, pos in rows[k + j]]
+        k += len(step)
+    U.assert_logits(np.concatenate(got), np.stack(exp), dtype == "float32")
