@@ -176,6 +176,18 @@ MIXERS_SIGNATURES = {
     "aphro_distance_bias_attention": (I, [P, L, P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, F, P, I, F,
                                           I, F, I, P, L, I, P]),
     "aphro_outer_memory_scan": (I, [P, P, L, P, L, P, L, P, P, L, P, P, P, P, I, P, P, P, I, L, I, I, I, I, P, F, F, I, I, P]),
+    "aphro_depth_residual_rms_norm": (I, [P, P, P, L, P, L, I, P, F, P, P, L, I, F, I, P]),
+    "aphro_poly_norm": (I, [P, P, L, L, I, F, F, F, F, F, I, P]),
+    "aphro_differential_norm_gate": (I, [P, L, P, L, P, L, L, I, I, I, F, F, F, I, P]),
+    "aphro_short_conv": (I, [P, L, P, P, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, I, P]),
+    "aphro_windowed_attention": (I, [P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, I, F, I, I, I, P, L, I, P]),
+    "aphro_experts_route": (I, [P, P, P, P, L, I, I, P]),
+    "aphro_experts_align_capacity": (L, [L, I]),
+    "aphro_experts_align": (I, [P, L, P, P, P, L, I, P]),
+    "aphro_experts_glu_gemm": (I, [P, P, L, P, P, P, P, L, I, I, I, F, F, I, P]),
+    "aphro_experts_down_gemm": (I, [P, P, P, P, P, P, L, I, I, I, I, P]),
+    "aphro_experts_combine": (I, [P, P, P, P, P, L, P, L, P, L, L, I, I, I, I, P]),
+    "aphro_clamped_glu": (I, [P, P, L, L, I, F, F, I, P]),
 }
 
 OK = 0

@@ -54,12 +54,15 @@ def _i32(t: torch.Tensor, n: int, what: str) -> None:
     _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n, f"{what}: int32 [{n}] expected")
 
 
-def embed_scale(table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
-    """fp32 residual rows ``table[ids] * scale``."""
-    _cuda(table, ids)
+def embed_scale(table: torch.Tensor, ids: torch.Tensor, scale: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 residual rows ``table[ids] * scale`` (into ``out`` fp32 [T, width] if given)."""
+    _cuda(table, ids, out)
     _need(table.dim() == 2 and table.is_contiguous() and ids.dtype == torch.int64 and ids.dim() == 1 and ids.is_contiguous(),
           "embed_scale: table [vocab, width] contiguous, ids int64 [T]")
-    out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+    if out is None:
+        out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (ids.shape[0], table.shape[1]),
+          "embed_scale: out fp32 [T, width], contiguous")
     check(_lib.mixers_lib().aphro_embed_scale_f32(out.data_ptr(), table.data_ptr(), ids.data_ptr(), ids.shape[0],
                                                   table.shape[1], table.shape[0], float(scale), _dt(table), _stream()),
           "embed_scale")
@@ -232,4 +235,205 @@ def outer_memory_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state, 
         state[1].data_ptr() if len(state) > 1 else None, state[2].data_ptr() if len(state) > 2 else None,
         slot_of_seq.data_ptr(), slots, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), S, T, heads, d, e, int(mode),
         _p(decay), float(q_scale), float(gate_cap), int(max_q_len), _dt(q), _stream()), "outer_memory_scan")
+    return out
+
+
+# ---- residual stream joined over depth, scalar-gain RMS norm, polynomial norm activation -------------------------------------
+def depth_residual_rms_norm(x_in: torch.Tensor, x_out: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None,
+                            history: Optional[torch.Tensor] = None, n_hist: int = 0, depth_w: Optional[torch.Tensor] = None,
+                            gain: float = 1.0, weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+                            dtype: Optional[torch.dtype] = None, want_out: bool = True) -> Optional[torch.Tensor]:
+    """r = x_in + y; with ``depth_w`` (fp32 [n_hist + 1]): history[n_hist] = r, r = sum_j depth_w[j] history[j];
+    x_out = r; returns rms_norm(r) * gain * weight in ``dtype`` (``want_out`` False: nothing).  x_in / x_out fp32 [T, W]
+    (may be the same tensor), history fp32 [entries, T, W]."""
+    T, W = x_in.shape
+    _cuda(x_in, x_out, y, history, depth_w, weight)
+    _need(x_in.dtype == torch.float32 and x_in.is_contiguous(), "depth_residual_rms_norm: x_in is fp32, contiguous")
+    _need(x_out is None or (x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == x_in.shape),
+          "depth_residual_rms_norm: x_out is fp32 [T, W], contiguous")
+    adt = dtype or (y.dtype if y is not None else (weight.dtype if weight is not None else None))
+    _need(adt in _DT, "depth_residual_rms_norm: the activation dtype is not given")
+    ys = 0
+    if y is not None:
+        _need(y.dtype == adt and y.shape[0] == T, "depth_residual_rms_norm: y [T, W] of the activation dtype")
+        ys = _rows(y, W, "depth_residual_rms_norm y")
+    hs = 0
+    if depth_w is not None:
+        _need(history is not None and history.dtype == torch.float32 and history.dim() == 3 and history.is_contiguous()
+              and tuple(history.shape[1:]) == (T, W) and 0 <= n_hist < history.shape[0],
+              "depth_residual_rms_norm: history fp32 [entries > n_hist, T, W]")
+        _need(depth_w.dtype == torch.float32 and depth_w.is_contiguous() and depth_w.numel() == n_hist + 1,
+              "depth_residual_rms_norm: depth_w fp32 [n_hist + 1]")
+        hs = history.stride(0)
+    _need(weight is None or (weight.dtype == adt and weight.numel() == W and weight.is_contiguous()),
+          "depth_residual_rms_norm: weight [W] of the activation dtype")
+    out = torch.empty(T, W, dtype=adt, device=x_in.device) if want_out else None
+    _need(out is not None or x_out is not None, "depth_residual_rms_norm: nothing to write")
+    check(_lib.mixers_lib().aphro_depth_residual_rms_norm(
+        x_in.data_ptr(), _p(x_out), _p(y), ys, _p(history) if depth_w is not None else None, hs, int(n_hist), _p(depth_w),
+        float(gain), _p(weight), _p(out), T, W, float(eps), _DT[adt], _stream()), "depth_residual_rms_norm")
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef, eps: float) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e per row, N = division by the row's root mean square; coef = (a, b, c, e) floats."""
+    _cuda(z)
+    _need(z.dim() == 2 and len(coef) == 4, "poly_norm: z [T, n], four coefficients")
+    T, n = z.shape
+    out = torch.empty(T, n, dtype=z.dtype, device=z.device)
+    check(_lib.mixers_lib().aphro_poly_norm(out.data_ptr(), z.data_ptr(), _rows(z, n, "poly_norm z"), T, n, float(coef[0]),
+                                            float(coef[1]), float(coef[2]), float(coef[3]), float(eps), _dt(z), _stream()),
+          "poly_norm")
+    return out
+
+
+def differential_norm_gate(out: torch.Tensor, a: torch.Tensor, gate: Optional[torch.Tensor], heads: int, maps: int, vdim: int,
+                           lam: float, out_scale: float, eps: float) -> None:
+    """out [T, heads * vdim] = out_scale * unit_rms_per_head(a_1 - lam a_2) * sigmoid(gate); a fp32 [T, heads * maps * vdim]."""
+    _cuda(out, a, gate)
+    T = a.shape[0]
+    _need(a.dtype == torch.float32 and out.shape == (T, heads * vdim), "differential_norm_gate: a fp32, out [T, heads * vdim]")
+    gs = 0
+    if gate is not None:
+        _need(gate.dtype == out.dtype and gate.shape == (T, heads * vdim), "differential_norm_gate: gate [T, heads * vdim]")
+        gs = _rows(gate, heads * vdim, "differential_norm_gate gate")
+    check(_lib.mixers_lib().aphro_differential_norm_gate(
+        out.data_ptr(), _rows(out, heads * vdim, "differential_norm_gate out"), a.data_ptr(),
+        _rows(a, heads * maps * vdim, "differential_norm_gate a"), _p(gate), gs, T, heads, maps, vdim, float(lam), float(out_scale),
+        float(eps), _dt(out), _stream()), "differential_norm_gate")
+
+
+def short_conv(u: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], state_slots: torch.Tensor, q_start: torch.Tensor,
+               q_len: torch.Tensor, ctx_len: torch.Tensor, seq_of_token: torch.Tensor, cq: int, ck: int = 0, cv: int = 0,
+               k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+               slot_mapping: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """Short causal convolution over time on the channels of u [T, cq + ck + cv] (dense rows, any row stride) with w
+    [channels, taps]; returns the first cq channels [T, cq]; the ck and cv channels go into the paged caches
+    (k_cache [blocks, block, ck], v_cache [blocks, block, cv] in any further split of the last axis) at ``slot_mapping``.
+    state [slots, taps - 1, channels] holds every request's last inputs and is advanced."""
+    _cuda(u, w, state, state_slots, q_start, q_len, ctx_len, seq_of_token, k_cache, v_cache, slot_mapping)
+    C = cq + ck + cv
+    T, S = u.shape[0], q_start.numel()
+    taps = w.shape[1]
+    _need(w.dim() == 2 and w.shape[0] == C and w.is_contiguous() and w.dtype == u.dtype, "short_conv: w [channels, taps]")
+    if taps > 1:
+        _need(state is not None and state.dtype == u.dtype and state.dim() == 3 and state.is_contiguous()
+              and tuple(state.shape[1:]) == (taps - 1, C), "short_conv: state [slots, taps - 1, channels]")
+    for t, nm in ((state_slots, "state_slots"), (q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    _i32(seq_of_token, T, "seq_of_token")
+    ncs = 0
+    if ck + cv:
+        _need(k_cache is not None and v_cache is not None and slot_mapping is not None and k_cache.is_contiguous()
+              and v_cache.is_contiguous() and k_cache.dtype == u.dtype == v_cache.dtype, "short_conv: caches of the activation dtype")
+        ncs = k_cache.shape[0] * k_cache.shape[1]
+        _need(k_cache.numel() == ncs * ck and v_cache.numel() == ncs * cv, "short_conv: cache rows do not fit the channels")
+        _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous(),
+              "short_conv: slots int64 [T]")
+    q = torch.empty(T, cq, dtype=u.dtype, device=u.device) if cq else None
+    check(_lib.mixers_lib().aphro_short_conv(
+        _p(q), cq, _p(k_cache) if ck + cv else None, _p(v_cache) if ck + cv else None, _p(slot_mapping) if ck + cv else None, ncs,
+        u.data_ptr(), _rows(u, C, "short_conv u"), w.data_ptr(), _p(state) if taps > 1 else None, state_slots.data_ptr(),
+        q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, cq, ck, cv, taps, _dt(u), _stream()),
+        "short_conv")
+    return q
+
+
+def windowed_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                       q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, seq_of_token: torch.Tensor, q_len_range,
+                       heads: int, maps: int, scale: float, window: int, keep_first: int, max_kv_len: int = 0) -> torch.Tensor:
+    """Every map's softmax attention under a sliding window that keeps the first tokens, fp32 [T, heads * maps * vdim].
+    q [T, heads * maps * dim]; k_cache [blocks, block, kv_heads * maps, dim], v_cache [blocks, block, kv_heads, vdim]."""
+    _cuda(q, k_cache, v_cache, block_tables, q_start, q_len, ctx_len, seq_of_token)
+    lo, hi = int(q_len_range[0]), int(q_len_range[1])
+    _need(0 < lo <= hi, "windowed_attention: q_len_range (shortest, longest)")
+    nb, bs, GM, d = k_cache.shape
+    G, e = v_cache.shape[2], v_cache.shape[3]
+    T, S = q.shape[0], q_start.numel()
+    _need(v_cache.shape[:2] == (nb, bs) and GM == G * maps and k_cache.is_contiguous() and v_cache.is_contiguous(),
+          "windowed_attention: cache shapes")
+    _need(q.dtype == k_cache.dtype == v_cache.dtype and heads % G == 0, "windowed_attention: one dtype, heads a multiple of kv heads")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.is_contiguous(),
+          "windowed_attention: block_tables int32 [S, max_blocks]")
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    _i32(seq_of_token, T, "seq_of_token")
+    out = torch.empty(T, heads * maps * e, dtype=torch.float32, device=q.device)
+    ws, ws_n = None, 0
+    check(_lib.mixers_lib().aphro_windowed_attention(
+        out.data_ptr(), heads * maps * e, q.data_ptr(), _rows(q, heads * maps * d, "windowed_attention q"), k_cache.data_ptr(),
+        v_cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(),
+        ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, lo, hi, heads, G, maps, d, e, float(scale), int(window), int(keep_first),
+        int(max_kv_len), _p(ws), ws_n, _dt(q), _stream()), "windowed_attention")
+    return out
+
+
+# ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------------
+def experts_route(router_out: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+    """router_out fp32 [T, outputs] -> (ids int32 [T, top], weights fp32 [T, top])."""
+    _cuda(router_out, correction)
+    T, R = router_out.shape
+    _need(router_out.dtype == torch.float32 and router_out.is_contiguous(), "experts_route: router outputs fp32, contiguous")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == R and correction.is_contiguous()),
+          "experts_route: correction fp32 [outputs]")
+    ids = torch.empty(T, top, dtype=torch.int32, device=router_out.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=router_out.device)
+    check(_lib.mixers_lib().aphro_experts_route(ids.data_ptr(), w.data_ptr(), router_out.data_ptr(), _p(correction), T, R, int(top),
+                                                _stream()), "experts_route")
+    return ids, w
+
+
+def experts_forward(h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                    limit: float, alpha: float, shared: Optional[torch.Tensor] = None,
+                    shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Weighted sum of every token's chosen experts.  h [T, W]; ids / weights [T, top]; w_gate_up [E, 2 ff, W] (gate rows, then
+    up rows), w_down [E, W, ff]; ids >= E are identity experts (their output is h).  ``shared`` [T, W] is added, times
+    sigmoid(shared_gate [T, 1])."""
+    _cuda(h, ids, weights, w_gate_up, w_down, shared, shared_gate)
+    T, W = h.shape
+    E, ff2, _ = w_gate_up.shape
+    ff, top = ff2 // 2, ids.shape[1]
+    lib = _lib.mixers_lib()
+    _need(w_gate_up.shape == (E, 2 * ff, W) and w_down.shape == (E, W, ff) and w_gate_up.is_contiguous() and w_down.is_contiguous()
+          and w_gate_up.dtype == h.dtype == w_down.dtype, "experts_forward: w_gate_up [E, 2 ff, W], w_down [E, W, ff] of h's dtype")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
+          and weights.shape == ids.shape and ids.shape[0] == T, "experts_forward: ids int32 / weights fp32 [T, top]")
+    hs = _rows(h, W, "experts_forward h")
+    cap = int(lib.aphro_experts_align_capacity(T * top, E))
+    dev = h.device
+    sorted_slots = torch.empty(cap, dtype=torch.int32, device=dev)
+    block_expert = torch.empty(cap // 16, dtype=torch.int32, device=dev)
+    num_blocks = torch.empty(1, dtype=torch.int32, device=dev)
+    y = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+    eo = torch.empty(T * top, W, dtype=torch.float32, device=dev)
+    out = torch.empty(T, W, dtype=h.dtype, device=dev)
+    st = _stream()
+    check(lib.aphro_experts_align(sorted_slots.data_ptr(), cap, block_expert.data_ptr(), num_blocks.data_ptr(), ids.data_ptr(),
+                                  T * top, E, st), "experts_align")
+    check(lib.aphro_experts_glu_gemm(y.data_ptr(), h.data_ptr(), hs, w_gate_up.data_ptr(), sorted_slots.data_ptr(),
+                                     block_expert.data_ptr(), num_blocks.data_ptr(), cap, top, ff, W, float(limit), float(alpha),
+                                     _dt(h), st), "experts_glu_gemm")
+    check(lib.aphro_experts_down_gemm(eo.data_ptr(), y.data_ptr(), w_down.data_ptr(), sorted_slots.data_ptr(),
+                                      block_expert.data_ptr(), num_blocks.data_ptr(), cap, top, W, ff, _dt(h), st),
+          "experts_down_gemm")
+    ss = sgs = 0
+    if shared is not None:
+        _need(shared.dtype == h.dtype and shared.shape == (T, W), "experts_forward: shared [T, W]")
+        ss = _rows(shared, W, "experts_forward shared")
+        if shared_gate is not None:
+            _need(shared_gate.dtype == h.dtype and shared_gate.shape == (T, 1), "experts_forward: shared_gate [T, 1]")
+            sgs = shared_gate.stride(0)
+    check(lib.aphro_experts_combine(out.data_ptr(), eo.data_ptr(), ids.data_ptr(), weights.data_ptr(), h.data_ptr(), hs, _p(shared),
+                                    ss, _p(shared_gate) if shared is not None else None, sgs, T, W, top, E, _dt(h), st),
+          "experts_combine")
+    return out
+
+
+def clamped_glu(x: torch.Tensor, d: int, limit: float, alpha: float) -> torch.Tensor:
+    """[T, >= 2 d] -> [T, d]: g = min(x[:, :d], limit), u = clamp(x[:, d:2d], +-limit), g * sigmoid(alpha g) * (u + 1)."""
+    _cuda(x)
+    _need(x.dim() == 2 and x.shape[1] >= 2 * d and x.stride(1) == 1, "clamped_glu: [T, >= 2 d] with dense rows")
+    out = torch.empty(x.shape[0], d, dtype=x.dtype, device=x.device)
+    check(_lib.mixers_lib().aphro_clamped_glu(out.data_ptr(), x.data_ptr(), x.stride(0) if x.shape[0] > 1 else max(x.stride(0), 2 * d),
+                                              x.shape[0], d, float(limit), float(alpha), _dt(x), _stream()), "clamped_glu")
     return out

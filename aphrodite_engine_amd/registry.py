@@ -52,6 +52,11 @@ def _register_builtin() -> None:
         from .fatudra import load_fatudra
         return load_fatudra(model_dir, config, **kw)
 
+    def gipozen(model_dir, config, **kw):
+        from .gipozen import load_gipozen
+        return load_gipozen(model_dir, config, **kw)
+
     for arch in ("LlamaForCausalLM", "MistralForCausalLM", "MixtralForCausalLM"):
         _LOADERS.setdefault(arch, llama)
     _LOADERS.setdefault("Fatudra", fatudra)
+    _LOADERS.setdefault("Gipozen", gipozen)

@@ -98,6 +98,86 @@ int aphro_outer_memory_scan(float* out, const void* q, int64_t q_stride, const v
                             int64_t num_tokens, int heads, int dim, int vdim, int mode, const float* decay, float q_scale,
                             float gate_cap, int max_q_len, int dtype, void* stream);
 
+/* ---- an fp32 residual stream joined over depth, scalar-gain RMS norm ---------------------------------------------------
+ * One launch, every step optional:
+ *   1. r = x_in + y                                       y [T, width] of `dtype` (row stride y_stride), NULL: r = x_in
+ *   2. history[n_hist] = r;  r = sum_{j <= n_hist} depth_w[j] * history[j]        (depth_w NULL: skipped)
+ *      history fp32 [.., T, width] with hist_stride elements between entries, depth_w fp32 [n_hist + 1]
+ *   3. x_out = r                                          fp32 [T, width], may be x_in; NULL: not written
+ *   4. out = r / sqrt(mean(r^2) + eps) * gain * weight    out [T, width] of `dtype`; weight [width] of `dtype` or NULL (ones) */
+int aphro_depth_residual_rms_norm(const float* x_in, float* x_out, const void* y, int64_t y_stride, float* history,
+                                  int64_t hist_stride, int n_hist, const float* depth_w, float gain, const void* weight,
+                                  void* out, int64_t num_tokens, int width, float eps, int dtype, void* stream);
+
+/* out[t, :] = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, N(v) = v / sqrt(mean(v^2) + eps) over the row.
+ * z [T, n] (row stride z_stride), out [T, n] contiguous, both of `dtype`; fp32 math, one rounding. */
+int aphro_poly_norm(void* out, const void* z, int64_t z_stride, int64_t num_tokens, int n, float a, float b, float c, float e,
+                    float eps, int dtype, void* stream);
+
+/* Joins the maps of a head: a fp32 [T, heads * maps * vdim] (head by head, map after map; maps 1 or 2),
+ *   o = a_1 - lambda * a_2  (maps == 1: o = a_1);  out = out_scale * o / sqrt(mean(o^2) + eps) * sigmoid(gate)
+ * with the mean over the head's vdim values; gate [T, heads * vdim] of `dtype` (NULL: none); out of `dtype`. */
+int aphro_differential_norm_gate(void* out, int64_t out_stride, const float* a, int64_t a_stride, const void* gate,
+                                 int64_t gate_stride, int64_t num_tokens, int heads, int maps, int vdim, float lambda,
+                                 float out_scale, float eps, int dtype, void* stream);
+
+/* Short causal convolution over time on each channel of u [T, cq + ck + cv] (row stride u_stride):
+ *   y_t[c] = sum_j w[c, j] * u_(t - taps + 1 + j)[c],  zeros before the sequence's start;  w [channels, taps] of `dtype`.
+ * Channels [0, cq) go to q_out [T, cq] (row stride); [cq, cq + ck) and the last cv go into the token-major paged caches
+ * k_cache [cache slots, ck] / v_cache [cache slots, cv] at row cache_slots[t] (int64; outside 0 .. num_cache_slots - 1: skipped).
+ * ck == cv == 0: no cache.  state [state slots, taps - 1, channels] of `dtype` holds each request's last taps - 1 inputs:
+ * read for the rows before a segment (never for positions before the sequence's start), rewritten afterwards.
+ * 1 <= taps <= 16. */
+int aphro_short_conv(void* q_out, int64_t q_out_stride, void* k_cache, void* v_cache, const int64_t* cache_slots,
+                     int64_t num_cache_slots, const void* u, int64_t u_stride, const void* w, void* state,
+                     const int32_t* state_slots, const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                     const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int cq, int ck, int cv, int taps, int dtype,
+                     void* stream);
+
+/* Softmax attention under a sliding window that keeps the first tokens: row i sees key j if j <= i and
+ * (i - j < window or j < keep_first); window <= 0: every earlier key.  No rotation, no bias.  A head carries `maps`
+ * attentions of their own over the same values: q [T, heads * maps * dim], k_cache [blocks, block_size, kv_heads * maps, dim],
+ * v_cache [blocks, block_size, kv_heads, vdim] of `dtype`; out fp32 [T, heads * maps * vdim], every map's normalised output.
+ * Segments as for aphro_distance_bias_attention.  bf16 with dim, vdim in {32, 64, 96, 128}: segments of 8 rows or more run on
+ * the matrix cores, shorter ones on the shared-key kernel (workspace as there); everything else on the fp32-math kernel. */
+int aphro_windowed_attention(float* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
+                             const void* v_cache, const int32_t* block_tables, int max_blocks, int64_t num_blocks,
+                             int block_size, const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                             const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int min_q_len, int max_q_len,
+                             int heads, int kv_heads, int maps, int dim, int vdim, float scale, int window, int keep_first,
+                             int max_kv_len, float* workspace, int64_t workspace_floats, int dtype, void* stream);
+
+/* ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------
+ * A SLOT is one (token, choice): slot = token * top + choice.
+ * moe_route: router_out fp32 [T, outputs] -> ids int32 [T, top], weights fp32 [T, top]: s = softmax(router_out); the top
+ *   values of s + correction (fp32 [outputs], NULL: none; ties to the lower index) are chosen, weights are their s. */
+int aphro_experts_route(int32_t* ids, float* weights, const float* router_out, const float* correction, int64_t num_tokens,
+                    int outputs, int top, void* stream);
+/* rows of sorted_slots that any step of num_slots slots over `experts` experts can need (a multiple of 16) */
+int64_t aphro_experts_align_capacity(int64_t num_slots, int experts);
+/* Sorts the slots whose id is below `experts` by expert into blocks of 16 rows (one expert per block, -1 pads a block):
+ * sorted_slots int32 [capacity], block_expert int32 [capacity / 16], num_blocks int32 [1].  Other ids are left out. */
+int aphro_experts_align(int32_t* sorted_slots, int64_t capacity, int32_t* block_expert, int32_t* num_blocks, const int32_t* ids,
+                    int64_t num_slots, int experts, void* stream);
+/* y[row, :] of `dtype` [capacity, ff], row = place in sorted_slots: g = min(W_gate h, limit), u = clamp(W_up h, +-limit),
+ * y = g * sigmoid(alpha * g) * (u + 1) with the block's expert; w_gate_up [experts, 2 * ff, width] (gate rows, then up rows);
+ * h [T, width] (row stride), the slot's token is slot / top.  Rows of padding are zero. */
+int aphro_experts_glu_gemm(void* y, const void* h, int64_t h_stride, const void* w_gate_up, const int32_t* sorted_slots,
+                       const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int ff, int width,
+                       float limit, float alpha, int dtype, void* stream);
+/* expert_out fp32 [slots, width]: row slot = W_down(expert) y[its sorted row]; w_down [experts, width, ff]. */
+int aphro_experts_down_gemm(float* expert_out, const void* y, const void* w_down, const int32_t* sorted_slots,
+                        const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int width, int ff,
+                        int dtype, void* stream);
+/* out[t] = sum_k weights[t, k] * (ids[t, k] < experts ? expert_out[t * top + k] : h[t])
+ *          + sigmoid(shared_gate[t]) * shared[t]        (shared NULL: none; shared_gate NULL: ungated; one number per row) */
+int aphro_experts_combine(void* out, const float* expert_out, const int32_t* ids, const float* weights, const void* h,
+                      int64_t h_stride, const void* shared, int64_t shared_stride, const void* shared_gate,
+                      int64_t shared_gate_stride, int64_t num_tokens, int width, int top, int experts, int dtype, void* stream);
+/* out[t, j] = g * sigmoid(alpha * g) * (u + 1), g = min(in[t, j], limit), u = clamp(in[t, d + j], +-limit), j < d */
+int aphro_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t num_tokens, int d, float limit, float alpha,
+                      int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
