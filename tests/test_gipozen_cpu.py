@@ -1,0 +1,118 @@
+"""CPU-side parts of the Gipozen integration: config checks, registry dispatch, checkpoint loading into the fused projections and
+the stacked expert weights, which layer owns which cache, and the plain restatement (oracle/gipozen.py) against itself where two
+formulations must agree."""
+import numpy as np
+import pytest
+import torch
+
+import gipozen_util as U
+from oracle import gipozen as O
+
+A = U.attention_layer
+
+
+def test_config_checks_layer_types_and_shared_keys():
+    from aphrodite_engine_amd.gipozen import GipozenConfig
+    layers = [A(), A(kv_from=0, mlp="moe"), A(mlp=None), A(kv_from=2)]
+    c = GipozenConfig.from_dict(U.make_config(layers))
+    assert len(c.layers) == 4 and c.logit_scale == 0.7 and c.eps == 1e-5
+    for bad in ([A(kv_from=0)], [A(), A(kv_from=0), A(kv_from=1)], [A(), A(kv_from=0, dim=16)], [A(), A(kv_from=3), A(), A()]):
+        with pytest.raises(ValueError):
+            GipozenConfig.from_dict(U.make_config(bad))
+    odd = U.make_config([A()])
+    odd["layers"][0]["type"] = "recurrent"
+    with pytest.raises(ValueError):
+        GipozenConfig.from_dict(odd)
+    odd = U.make_config([A()])
+    odd["layers"][0]["mlp"]["kind"] = "sparse"
+    with pytest.raises(ValueError):
+        GipozenConfig.from_dict(odd)
+
+
+def test_registry_knows_the_design():
+    from aphrodite_engine_amd import registry
+    assert "Gipozen" in registry.supported_architectures()
+    assert registry.architecture_of({"architecture": "Gipozen"}) == "Gipozen"
+
+
+def test_checkpoint_fills_fused_projections_experts_and_caches(tmp_path):
+    from aphrodite_engine_amd.loader import load_model
+    cfg = U.make_config([A(), A(kv_from=0, taps=2, mlp="moe"), A(heads=3, kv_heads=3, dim=16, vdim=24, mlp=None),
+                         A(kv_from=0, mlp="moe", identity=0, shared_ff=0)])
+    W = U.make_weights(cfg, seed=3)
+    U.write_checkpoint(str(tmp_path), cfg, W)
+    m = load_model(str(tmp_path), dtype=torch.float32, device="cpu")
+    assert type(m).__name__ == "GipozenForCausalLM"
+    for i, layer in enumerate(m.layers):
+        mix, a, at = layer.mix, layer.mix.attn, 0
+        assert mix.names == (["q", "k", "v", "g"] if a.own_kv else ["q", "g"])
+        for name, n in zip(mix.names, mix.splits):
+            np.testing.assert_array_equal(mix.in_proj.weight[at:at + n].numpy(), W[f"l{i}.mix.{name}"])
+            if name != "g":
+                np.testing.assert_array_equal(a.conv[at:at + n].numpy(), W[f"l{i}.mix.{name}.conv"])
+            at += n
+        assert float(mix.in_proj.weight[at:].abs().sum()) == 0.0 and mix.in_proj.weight.shape[0] % 8 == 0
+        want = O.differential_lambda(W[f"l{i}.mix.lq1"], W[f"l{i}.mix.lk1"], W[f"l{i}.mix.lq2"], W[f"l{i}.mix.lk2"], a.diff)
+        assert abs(a.lam - want) < 1e-5
+        assert layer.gain1 == float(W[f"l{i}.norm1"]) and layer.dwa.numel() == i + 2
+    # layers 1 and 3 read layer 0's pages; every layer has a convolution state of its own
+    assert m.kv_index == [0, 0, 3, 0] and m.state_index == [1, 2, 4, 5] and len(m.specs) == 6
+    e = m.layers[1].mlp
+    np.testing.assert_array_equal(e.w_gate_up[2, :e.ff].numpy(), W["l1.mlp.e2.gate"])
+    np.testing.assert_array_equal(e.w_gate_up[2, e.ff:].numpy(), W["l1.mlp.e2.up"])
+    np.testing.assert_array_equal(e.w_down[4].numpy(), W["l1.mlp.e4.down"])
+    np.testing.assert_array_equal(e.shared_in.weight[2 * e.shared_ff].numpy(), W["l1.mlp.shared.sg"][0])
+    assert e.router.dtype == torch.float32 and e.router.shape[0] == e.experts + e.identity
+    assert m.layers[3].mlp.shared_ff == 0 and m.layers[2].mlp is None
+    caches = m.make_caches(7, 16, 3, "cpu")
+    assert caches[0][0].shape == (7, 16, 4, 24) and caches[0][1].shape == (7, 16, 2, 40) and caches[2].shape == (3, 1, 6 * 2 * 24)
+    # a tensor too many, one missing, one of the wrong shape
+    for change in ("extra", "missing", "shape"):
+        W2 = dict(W)
+        if change == "extra":
+            W2["l1.mix.k"] = W["l0.mix.k"]
+        elif change == "missing":
+            del W2["l3.dwa"]
+        else:
+            W2["l2.mix.q.conv"] = W["l2.mix.q.conv"][:, :2]
+        U.write_checkpoint(str(tmp_path / change), cfg, W2)
+        with pytest.raises(ValueError):
+            load_model(str(tmp_path / change), dtype=torch.float32, device="cpu")
+
+
+def test_restatement_mask_convolution_and_average():
+    assert [j for j in range(10) if O.visible(9, j, 3, 2)] == [0, 1, 7, 8, 9]
+    assert [j for j in range(10) if O.visible(9, j, 3, 0)] == [7, 8, 9]
+    assert [j for j in range(4) if O.visible(2, j, 100, 0)] == [0, 1, 2]
+    u = np.arange(12, dtype=np.float64).reshape(6, 2)
+    w = np.array([[1.0, 10.0, 100.0], [0.0, 0.0, 1.0]])
+    y = O.short_causal_conv(u, w)
+    assert y[0, 0] == 100 * u[0, 0] and y[2, 0] == u[0, 0] + 10 * u[1, 0] + 100 * u[2, 0]
+    np.testing.assert_array_equal(y[:, 1], u[:, 1])                # the last tap is the current token
+    X = [np.full((2, 3), float(i + 1)) for i in range(3)]
+    np.testing.assert_allclose(O.depth_average(X, [0.5, 0.25, 2.0]), np.full((2, 3), 0.5 + 0.5 + 6.0))
+
+
+def test_restatement_window_attention_equals_a_masked_matrix_form():
+    rng = np.random.default_rng(0)
+    T, d, e = 40, 8, 5
+    q, k, v = rng.standard_normal((T, d)), rng.standard_normal((T, d)), rng.standard_normal((T, e))
+    for window, keep in ((7, 2), (100, 0), (1, 0), (3, 3)):
+        s = q @ k.T * 0.3
+        mask = np.array([[O.visible(i, j, window, keep) for j in range(T)] for i in range(T)])
+        s = np.where(mask, s, -np.inf)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        np.testing.assert_allclose(O.windowed_softmax_attention(q, k, v, 0.3, window, keep), (p / p.sum(-1, keepdims=True)) @ v,
+                                   rtol=1e-10, atol=1e-12)
+
+
+def test_restatement_router_and_identity_experts():
+    h = np.array([[1.0, 0.0, 0.0], [0.0, 2.0, 0.0]])
+    router = np.eye(3)
+    idx, w = O.route(h, router, np.array([0.0, 0.0, 5.0]), 2)
+    assert idx[0].tolist() == [2, 0] and idx[1].tolist() == [2, 1]
+    s = np.exp(h[0]) / np.exp(h[0]).sum()
+    np.testing.assert_allclose(w[0], [s[2], s[0]])                 # the correction chooses, the plain score weighs
+    mc = {"router": {"experts": 0, "identity": 3, "top": 3}, "expert": {"limit": 1.0}}
+    out = O.moe_ff(h, {"router": router, "correction": np.zeros(3)}, "", mc)
+    np.testing.assert_allclose(out, h)                             # all weights sum to one, every expert returns h
