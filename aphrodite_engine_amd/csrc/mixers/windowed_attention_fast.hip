@@ -1,0 +1,568 @@
+// bf16 fast paths of differential attention under a sliding window that keeps the first tokens (same semantics as
+// windowed_attention.hip followed by differential_norm_gate, in one launch: the two maps of a head are computed side by side,
+// joined as a_1 - lambda a_2, brought to unit RMS over the head's values, scaled and gated, and leave as bf16):
+//
+//  * wa_prefill_kernel<DK, DV>: segments of >= WA_MFMA_MIN_LEN rows.  A workgroup of four waves owns 64 consecutive query rows
+//    of one (segment, head) and BOTH maps: per key tile of 64 it stages the two maps' key rows and the one shared value tile in
+//    LDS (K chunk-swizzled, V transposed, the next tile's cache rows in flight in registers meanwhile), S^T = K Q^T on
+//    v_mfma_f32_16x16x32_bf16 for each map, so that the probabilities come out as the B operand of O^T = V^T P^T and the V
+//    fragments read from LDS feed both maps.  Only key tiles that some row of the workgroup can see are visited: the tiles of the
+//    kept first tokens, then from the tile of the lowest window start on; a wave skips tiles none of its 16 rows sees, and the
+//    mask is applied only on tiles that are not wholly visible to the wave.
+//  * wa_decode_kernel<QHM, CHL>: the other rows (single decoded tokens, short portions), one workgroup per (row, kv head, group
+//    of QHM / 2 query heads): one pass over the row's visible keys -- numbered kept tokens first, then the window -- with a key
+//    row read by 2^CHL lanes x 16 bytes, partial dot products folded with DPP moves, each value row used by all QHM (head, map)
+//    pairs; four waves take the steps round-robin and merge through LDS, where the maps are then joined, normed and gated.
+#include "mixers_common.h"
+
+namespace aphro {
+
+struct WAParams {
+  uint16_t* out;              // bf16 [T, heads * vdim]
+  const uint16_t* q;          // bf16 [T, heads * 2 * dim]
+  const uint16_t* gate;       // bf16 [T, heads * vdim] raw, or null
+  const uint16_t* k_cache;    // [blocks, block, kv_heads * 2, dim]
+  const uint16_t* v_cache;    // [blocks, block, kv_heads, vdim]
+  const int32_t* block_tables;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* ctx_len;
+  const int32_t* seq_of_token;
+  int64_t out_stride, q_stride, gate_stride, num_blocks;
+  int max_blocks, block_size, heads, kv_heads, dim, vdim, window, keep_first, min_len, bs_shift, max_tiles;
+  float scale, lambda, out_scale, eps;
+};
+
+__device__ __forceinline__ int wa_slot(const WAParams& p, const int32_t* bt, int key) {
+  int blk, off;
+  if (p.bs_shift >= 0) {
+    blk = bt[key >> p.bs_shift];
+    off = key & (p.block_size - 1);
+  } else {
+    blk = bt[key / p.block_size];
+    off = key % p.block_size;
+  }
+  if (blk < 0 || blk >= p.num_blocks) blk = 0;             // never read outside the pool
+  return blk * p.block_size + off;
+}
+
+constexpr int WA_BM = 64, WA_BN = 64, WA_VT = WA_BN + 4;
+
+template <int DK, int DV>
+struct WAStage {
+  static constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  static constexpr int KI = (WA_BN * NCHK + 255) / 256, VI = (WA_BN / 2 * NCHV + 255) / 256;
+  u16x8 k[2][KI], v0[VI], v1[VI];
+};
+
+template <int DK, int DV>
+__device__ __forceinline__ void wa_load(WAStage<DK, DV>& st, const WAParams& p, const int32_t* bt, int kvh, int t0, int nk) {
+  constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  const int64_t krow = (int64_t)p.kv_heads * 2 * DK, vrow = (int64_t)p.kv_heads * DV;
+#pragma unroll
+  for (int it = 0; it < WAStage<DK, DV>::KI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < WA_BN * NCHK) {
+      const int tok = i / NCHK, ch = i % NCHK;
+      const uint16_t* kr = p.k_cache + (int64_t)wa_slot(p, bt, min(t0 + tok, nk - 1)) * krow + (int64_t)kvh * 2 * DK + 8 * ch;
+      st.k[0][it] = *reinterpret_cast<const u16x8*>(kr);
+      st.k[1][it] = *reinterpret_cast<const u16x8*>(kr + DK);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < WAStage<DK, DV>::VI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < WA_BN / 2 * NCHV) {
+      const int tp = i / NCHV, ch = i % NCHV;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int key = min(t0 + 2 * tp + half, nk - 1);
+        u16x8 vv = *reinterpret_cast<const u16x8*>(p.v_cache + (int64_t)wa_slot(p, bt, key) * vrow + kvh * DV + 8 * ch);
+        if (t0 + 2 * tp + half >= nk) vv = u16x8{0, 0, 0, 0, 0, 0, 0, 0};    // beyond the sequence: no NaN into P V
+        if (half == 0) st.v0[it] = vv;
+        else st.v1[it] = vv;
+      }
+    }
+  }
+}
+
+template <int DK, int DV>
+__device__ __forceinline__ void wa_store(const WAStage<DK, DV>& st, uint16_t* k_lds, uint16_t* vt_lds) {
+  constexpr int NCHK = DK / 8, NCHV = DV / 8;
+  constexpr int SWZ = (NCHK & -NCHK) - 1;
+#pragma unroll
+  for (int it = 0; it < WAStage<DK, DV>::KI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < WA_BN * NCHK) {
+      const int tok = i / NCHK, ch = i % NCHK;
+      *reinterpret_cast<u16x8*>(&k_lds[tok * DK + 8 * (ch ^ (tok & SWZ))]) = st.k[0][it];
+      *reinterpret_cast<u16x8*>(&k_lds[WA_BN * DK + tok * DK + 8 * (ch ^ (tok & SWZ))]) = st.k[1][it];
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < WAStage<DK, DV>::VI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < WA_BN / 2 * NCHV) {
+      const int tp = i / NCHV, ch = i % NCHV;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<uint32_t*>(&vt_lds[(8 * ch + j) * WA_VT + 2 * tp]) = (uint32_t)st.v0[it][j] | ((uint32_t)st.v1[it][j] << 16);
+    }
+  }
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void wa_prefill_kernel(WAParams p) {
+  constexpr int NCHK = DK / 8, NKS = DK / 32, NDT = DV / 16, NH = WA_BN / 16, NPK = WA_BN / 32;
+  constexpr int SWZ = (NCHK & -NCHK) - 1;
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2 * WA_BN * DK];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DV * WA_VT];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  const int seq = blockIdx.y;
+  const int len = p.q_len[seq];
+  if (len < p.min_len) return;
+  const int ntiles = (len + WA_BM - 1) / WA_BM;
+  // Workgroups go to the 8 XCDs round-robin by their linear index and each XCD has its own L2: the (tile, head) pairs are
+  // numbered so that the query heads of one kv head -- the workgroups that read the same keys and values -- share an XCD.
+  int head, rank;
+  {
+    constexpr int NX = 8;
+    const int G = p.kv_heads, QU = p.heads / p.kv_heads, x = blockIdx.x % NX, j = blockIdx.x / NX;
+    if (G % NX == 0) {
+      const int ux = (G / NX) * QU, ul = j % ux;
+      rank = j / ux;
+      head = ((ul / QU) * NX + x) * QU + ul % QU;
+    } else if (NX % G == 0) {
+      const int share = NX / G, pair = j * share + x / G;
+      rank = pair / QU;
+      head = (x % G) * QU + pair % QU;
+    } else {
+      rank = blockIdx.x / p.heads;
+      head = blockIdx.x % p.heads;
+    }
+  }
+  const int tile = ntiles - 1 - rank;
+  if (tile < 0 || rank >= p.max_tiles) return;
+  const int ctx = p.ctx_len[seq], s0 = p.q_start[seq];
+  const int kvh = head / (p.heads / p.kv_heads);
+  const int q0 = tile * WA_BM;
+  const int qrow = q0 + 16 * wave + c;
+  const bool qvalid = qrow < len;
+  const int qpos = ctx + qrow;
+  const int window = p.window > 0 ? p.window : 0x3fffffff, keep = p.keep_first;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float qs = p.scale * LOG2E;                        // scores in units of ln 2: the exponentials are exp2
+  u32x4 qf[2][NKS];
+  {
+    const uint16_t* qp = p.q + (int64_t)(s0 + min(qrow, len - 1)) * p.q_stride + (int64_t)head * 2 * DK;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) qf[t][ks] = *reinterpret_cast<const u32x4*>(qp + t * DK + 32 * ks + 8 * g);
+  }
+  f32x4 o[2][NDT];
+  float m_run[2], l_run[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    m_run[t] = -INFINITY;
+    l_run[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) o[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  const int nk = ctx + min(len, q0 + WA_BM);               // keys the tile's last row sees
+  const int lo_wg = max(0, ctx + q0 - window + 1);         // the lowest window start among the workgroup's rows
+  const int win_tile = lo_wg / WA_BN * WA_BN;
+  const int pw0 = ctx + q0 + 16 * wave, pw1 = pw0 + 15;    // positions of the wave's rows
+
+  WAStage<DK, DV> st;
+  int t0 = keep > 0 ? 0 : win_tile;
+  wa_load<DK, DV>(st, p, bt, kvh, t0, nk);
+  while (t0 < nk) {
+    int t_next = t0 + WA_BN;
+    if (t_next >= keep && t_next < win_tile) t_next = win_tile;        // past the kept tokens: on to the window
+    __syncthreads();                                        // the previous tile is consumed
+    wa_store<DK, DV>(st, k_lds, vt_lds);
+    __syncthreads();
+    if (t_next < nk) wa_load<DK, DV>(st, p, bt, kvh, t_next, nk);      // in flight during this tile's products
+    const int tc = t0;
+    t0 = t_next;
+    if (tc > pw1) continue;                                 // every key of the tile is ahead of the wave's rows
+    if (tc >= keep && tc + WA_BN - 1 < pw0 - window + 1) continue;     // ... or behind every row's window, none of them kept
+    f32x4 s[2][NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const int tok = 16 * h + c;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          const int ch = (4 * ks + g) ^ (tok & SWZ);
+          const u32x4 kf = *reinterpret_cast<const u32x4*>(&k_lds[t * WA_BN * DK + tok * DK + 8 * ch]);
+          s[t][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[t][ks]),
+                                                            s[t][h], 0, 0, 0);
+        }
+      }
+    }
+    // wholly visible to the wave: behind its first row and inside its last row's window
+    const bool masked = !(tc + WA_BN - 1 <= pw0 && pw1 - tc < window);
+    u32x4 pf[2][NPK];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float pv[NH][4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float xv = s[t][h][r] * qs;
+          if (masked) {
+            const int j = tc + 16 * h + 4 * g + r;
+            xv = (j <= qpos && (qpos - j < window || j < keep)) ? xv : -INFINITY;
+          }
+          pv[h][r] = xv;
+          mx = fmaxf(mx, xv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[t], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;          // a row that has seen no key yet
+      const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_safe);
+      m_run[t] = m_new;
+      float lsum = 0.f;
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float e = __builtin_amdgcn_exp2f(pv[h][r] - m_safe);  // a masked score is -inf: exactly 0
+          pv[h][r] = e;
+          lsum += e;
+        }
+      l_run[t] = l_run[t] * alpha + lsum;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) o[t][dt] *= alpha;
+#pragma unroll
+      for (int pk = 0; pk < NPK; ++pk)
+        pf[t][pk] = u32x4{pack2_16<true>(pv[2 * pk][0], pv[2 * pk][1]), pack2_16<true>(pv[2 * pk][2], pv[2 * pk][3]),
+                          pack2_16<true>(pv[2 * pk + 1][0], pv[2 * pk + 1][1]), pack2_16<true>(pv[2 * pk + 1][2], pv[2 * pk + 1][3])};
+    }
+#pragma unroll
+    for (int pk = 0; pk < NPK; ++pk) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const uint16_t* vr = &vt_lds[(16 * dt + c) * WA_VT + 32 * pk + 4 * g];
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[t][pk]),
+                                                             o[t][dt], 0, 0, 0);
+      }
+    }
+  }
+  // join the maps: the row's DV values sit in the four lanes c, c + 16, c + 32, c + 48
+  float inv[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    float l = l_run[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    inv[t] = l > 0.f ? 1.f / l : 0.f;
+  }
+  const float f1 = p.lambda * inv[1];
+  float ss = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float d = o[0][dt][r] * inv[0] - f1 * o[1][dt][r];
+      o[0][dt][r] = d;
+      ss += d * d;
+    }
+  ss += __shfl_xor(ss, 16, 64);
+  ss += __shfl_xor(ss, 32, 64);
+  if (!qvalid) return;
+  const float rstd = p.out_scale / sqrtf(ss / (float)DV + p.eps);
+  uint16_t* op = p.out + (int64_t)(s0 + qrow) * p.out_stride + head * DV + 4 * g;
+  const uint16_t* gp = p.gate ? p.gate + (int64_t)(s0 + qrow) * p.gate_stride + head * DV + 4 * g : nullptr;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = o[0][dt][r] * rstd;
+    if (gp) {
+      const u16x4 gg = *reinterpret_cast<const u16x4*>(gp + 16 * dt);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] *= sigmoid_f(BFloat::to_f32(gg[r]));
+    }
+    *reinterpret_cast<u32x2*>(op + 16 * dt) = u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
+  }
+}
+
+// QHM (head, map) pairs = QHM / 2 query heads of one kv head per workgroup
+template <int QHM, int CHL>
+__global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
+  constexpr int CH = 1 << CHL;       // lanes per key row (16 bytes each)
+  constexpr int KP = 64 / CH;        // keys per load instruction
+  constexpr int NI = 4;              // load instructions per step of the online softmax
+  constexpr int KT = NI * KP;        // keys per step
+  constexpr int NHQ = QHM / 2;       // query heads of the workgroup
+  __shared__ float merge[4][QHM][2 + 8 * CH];
+  __shared__ float fin[QHM][8 * CH];
+  const int t = blockIdx.x, kvh = blockIdx.y;
+  const int seq = p.seq_of_token[t];
+  if (p.q_len[seq] >= p.min_len) return;                   // the prompt kernel's share
+  const int pos = p.ctx_len[seq] + (t - p.q_start[seq]);
+  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int ns = min(p.keep_first, lo);
+  const int nvis = ns + pos - lo + 1;                      // visible keys: [0, ns) and [lo, pos]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ck = lane & (CH - 1), kg = lane >> CHL;
+  const bool kin = 8 * ck < p.dim, vin = 8 * ck < p.vdim;
+  const int head0 = kvh * (p.heads / p.kv_heads) + blockIdx.z * NHQ;
+  float qv[QHM][8];
+#pragma unroll
+  for (int qh = 0; qh < QHM; ++qh) {
+    u16x8 raw = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (kin) raw = *reinterpret_cast<const u16x8*>(p.q + (int64_t)t * p.q_stride + ((int64_t)head0 * 2 + qh) * p.dim + 8 * ck);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qv[qh][j] = BFloat::to_f32(raw[j]);
+  }
+  const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  const int64_t krow = (int64_t)p.kv_heads * 2 * p.dim, vrow = (int64_t)p.kv_heads * p.vdim;
+  float m[QHM], l[QHM], acc[QHM][8];
+#pragma unroll
+  for (int qh = 0; qh < QHM; ++qh) {
+    m[qh] = -INFINITY;
+    l[qh] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[qh][j] = 0.f;
+  }
+  const int ntiles = (nvis + KT - 1) / KT;
+  for (int tile = wave; tile < ntiles; tile += 4) {
+    float sc[NI][QHM];
+    u16x8 vv[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = tile * KT + i * KP + kg;
+      const bool valid = r < nvis;
+      const int key = valid ? (r < ns ? r : lo + (r - ns)) : 0;
+      const int64_t slot = wa_slot(p, bt, key);
+      u16x8 k0 = u16x8{0, 0, 0, 0, 0, 0, 0, 0}, k1 = k0;
+      vv[i] = k0;
+      if (valid && kin) {
+        const uint16_t* kr = p.k_cache + slot * krow + (int64_t)kvh * 2 * p.dim + 8 * ck;
+        k0 = *reinterpret_cast<const u16x8*>(kr);
+        k1 = *reinterpret_cast<const u16x8*>(kr + p.dim);
+      }
+      if (valid && vin) vv[i] = *reinterpret_cast<const u16x8*>(p.v_cache + slot * vrow + kvh * p.vdim + 8 * ck);
+      float kf[2][8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        kf[0][j] = BFloat::to_f32(k0[j]);
+        kf[1][j] = BFloat::to_f32(k1[j]);
+      }
+#pragma unroll
+      for (int qh = 0; qh < QHM; ++qh) {
+        float d = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) d += qv[qh][j] * kf[qh & 1][j];
+        d = group_sum<CHL>(d);
+        sc[i][qh] = valid ? d * p.scale : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int qh = 0; qh < QHM; ++qh) {
+      float mx = sc[0][qh];
+#pragma unroll
+      for (int i = 1; i < NI; ++i) mx = fmaxf(mx, sc[i][qh]);
+#pragma unroll
+      for (int o = CH; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_new = fmaxf(m[qh], mx);                // finite: the tile's first key exists
+      const float alpha = (m[qh] == -INFINITY) ? 0.f : __expf(m[qh] - m_new);
+      m[qh] = m_new;
+      float ls = 0.f;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const float e = (sc[i][qh] == -INFINITY) ? 0.f : __expf(sc[i][qh] - m_new);
+        sc[i][qh] = e;
+        ls += e;
+      }
+      l[qh] = l[qh] * alpha + ls;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[qh][j] *= alpha;
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float vf = BFloat::to_f32(vv[i][j]);
+#pragma unroll
+        for (int qh = 0; qh < QHM; ++qh) acc[qh][j] += sc[i][qh] * vf;
+      }
+    }
+  }
+  // fold the key groups of the wave, then the four waves
+#pragma unroll
+  for (int qh = 0; qh < QHM; ++qh) {
+#pragma unroll
+    for (int o = CH; o < 64; o <<= 1) {
+      l[qh] += __shfl_xor(l[qh], o, 64);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[qh][j] += __shfl_xor(acc[qh][j], o, 64);
+    }
+    if (lane == 0) {
+      merge[wave][qh][0] = m[qh];
+      merge[wave][qh][1] = l[qh];
+    }
+    if (kg == 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) merge[wave][qh][2 + 8 * ck + j] = acc[qh][j];
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < QHM * p.vdim; idx += 256) {
+    const int qh = idx / p.vdim, col = idx % p.vdim;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, merge[w][qh][0]);
+    float L = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = (merge[w][qh][0] == -INFINITY) ? 0.f : __expf(merge[w][qh][0] - M);
+      L += merge[w][qh][1] * f;
+      o += merge[w][qh][2 + col] * f;
+    }
+    fin[qh][col] = o / L;
+  }
+  __syncthreads();
+  if (wave >= NHQ) return;
+  const int head = head0 + wave;
+  float ss = 0.f;
+  for (int col = lane; col < p.vdim; col += 64) {
+    const float d = fin[2 * wave][col] - p.lambda * fin[2 * wave + 1][col];
+    ss += d * d;
+  }
+  const float rstd = p.out_scale / sqrtf(wave_sum(ss) / (float)p.vdim + p.eps);
+  for (int col = lane; col < p.vdim; col += 64) {
+    float d = (fin[2 * wave][col] - p.lambda * fin[2 * wave + 1][col]) * rstd;
+    if (p.gate) d *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head * p.vdim + col]));
+    p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(d);
+  }
+}
+
+template <int DK>
+static void wa_launch_prefill_dv(const WAParams& p, dim3 grid, hipStream_t st) {
+  switch (p.vdim) {
+    case 32: hipLaunchKernelGGL((wa_prefill_kernel<DK, 32>), grid, dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((wa_prefill_kernel<DK, 64>), grid, dim3(256), 0, st, p); break;
+    case 96: hipLaunchKernelGGL((wa_prefill_kernel<DK, 96>), grid, dim3(256), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((wa_prefill_kernel<DK, 128>), grid, dim3(256), 0, st, p); break;
+  }
+}
+
+static bool wa_prefill_supported(int dim, int vdim) {
+  auto ok = [](int d) { return d == 32 || d == 64 || d == 96 || d == 128; };
+  return ok(dim) && ok(vdim);
+}
+
+static void wa_prefill_launch(const WAParams& p0, int max_q_len, int num_seqs, hipStream_t st) {
+  WAParams p = p0;
+  p.max_tiles = (max_q_len + WA_BM - 1) / WA_BM;
+  const int per_seq = (p.max_tiles * p.heads + 7) / 8 * 8;   // a multiple of the XCD count: the numbering repeats per segment
+  const dim3 grid((unsigned)per_seq, (unsigned)num_seqs);
+  switch (p.dim) {
+    case 32: wa_launch_prefill_dv<32>(p, grid, st); break;
+    case 64: wa_launch_prefill_dv<64>(p, grid, st); break;
+    case 96: wa_launch_prefill_dv<96>(p, grid, st); break;
+    case 128: wa_launch_prefill_dv<128>(p, grid, st); break;
+  }
+}
+
+static int wa_decode_chl(int dim, int vdim) {
+  const int pieces = (max(dim, vdim) + 7) / 8;
+  int chl = 2;
+  while ((1 << chl) < pieces) ++chl;
+  return chl;
+}
+
+// (head, map) pairs per workgroup: 4 where the kv head has an even number of query heads and the row fits, else 2
+static int wa_decode_qhm(int heads, int kv_heads, int dim, int vdim) {
+  const int chl = wa_decode_chl(dim, vdim);
+  if ((dim & 7) || (vdim & 7) || chl > 5) return 0;
+  if ((heads / kv_heads) % 2 == 0 && 4 * (1 << chl) <= 64) return 4;
+  return 2;
+}
+
+static void wa_decode_launch(const WAParams& p, int64_t num_tokens, hipStream_t st) {
+  const int qhm = wa_decode_qhm(p.heads, p.kv_heads, p.dim, p.vdim), chl = wa_decode_chl(p.dim, p.vdim);
+  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)(p.heads / p.kv_heads / (qhm / 2)));
+#define WDEC(QHM, CHL) hipLaunchKernelGGL((wa_decode_kernel<QHM, CHL>), grid, dim3(256), 0, st, p)
+  if (qhm == 4) {
+    switch (chl) {
+      case 2: WDEC(4, 2); break;
+      case 3: WDEC(4, 3); break;
+      case 4: WDEC(4, 4); break;
+    }
+  } else {
+    switch (chl) {
+      case 2: WDEC(2, 2); break;
+      case 3: WDEC(2, 3); break;
+      case 4: WDEC(2, 4); break;
+      case 5: WDEC(2, 5); break;
+    }
+  }
+#undef WDEC
+}
+
+constexpr int WA_MFMA_MIN_LEN = 8;
+
+}  // namespace aphro
+
+using namespace aphro;
+
+/* 1 if aphro_differential_window_attention serves these sizes (bf16 only), else 0 */
+extern "C" int aphro_differential_window_attention_supported(int heads, int kv_heads, int dim, int vdim, int dtype) {
+  if (dtype != APHRO_BF16 || heads <= 0 || kv_heads <= 0 || heads % kv_heads) return 0;
+  return wa_decode_qhm(heads, kv_heads, dim, vdim) != 0 && wa_prefill_supported(dim, vdim) ? 1 : 0;
+}
+
+extern "C" int aphro_differential_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
+                                                   int64_t gate_stride, const void* k_cache, const void* v_cache,
+                                                   const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size,
+                                                   const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                                                   const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int min_q_len,
+                                                   int max_q_len, int heads, int kv_heads, int dim, int vdim, float scale, int window,
+                                                   int keep_first, float lambda, float out_scale, float eps, int dtype, void* stream) {
+  if (num_tokens == 0) return APHRO_OK;
+  APHRO_CHECK(out && q && k_cache && v_cache && block_tables && q_start && q_len && ctx_len && seq_of_token,
+              "differential_window_attention: null argument");
+  APHRO_CHECK(aphro_differential_window_attention_supported(heads, kv_heads, dim, vdim, dtype),
+              "differential_window_attention: bf16 with dim, vdim in {32, 64, 96, 128} only (heads %d / %d, dim %d, vdim %d, dtype %d)",
+              heads, kv_heads, dim, vdim, dtype);
+  APHRO_CHECK(block_size > 0 && max_blocks > 0 && num_blocks > 0 && num_seqs > 0 && keep_first >= 0 && 0 < min_q_len &&
+                  min_q_len <= max_q_len, "differential_window_attention: bad geometry");
+  APHRO_CHECK(q_stride >= (int64_t)heads * 2 * dim && out_stride >= (int64_t)heads * vdim && (!gate || gate_stride >= (int64_t)heads * vdim),
+              "differential_window_attention: row strides smaller than the rows");
+  APHRO_CHECK(((uintptr_t)q & 15) == 0 && (q_stride & 7) == 0 && ((uintptr_t)out & 7) == 0 && (out_stride & 3) == 0 &&
+                  ((uintptr_t)gate & 7) == 0 && (gate_stride & 3) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0,
+              "differential_window_attention: rows must be 16-byte aligned (q, caches) and 8-byte aligned (out, gate)");
+  WAParams p;
+  p.out = (uint16_t*)out; p.q = (const uint16_t*)q; p.gate = (const uint16_t*)gate;
+  p.k_cache = (const uint16_t*)k_cache; p.v_cache = (const uint16_t*)v_cache;
+  p.block_tables = block_tables; p.q_start = q_start; p.q_len = q_len; p.ctx_len = ctx_len; p.seq_of_token = seq_of_token;
+  p.out_stride = out_stride; p.q_stride = q_stride; p.gate_stride = gate_stride; p.num_blocks = num_blocks;
+  p.max_blocks = max_blocks; p.block_size = block_size; p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim;
+  p.window = window; p.keep_first = keep_first; p.scale = scale; p.lambda = lambda; p.out_scale = out_scale; p.eps = eps;
+  p.max_tiles = 0;
+  p.bs_shift = -1;
+  for (int sft = 0; sft < 20; ++sft)
+    if ((1 << sft) == block_size) p.bs_shift = sft;
+  p.min_len = WA_MFMA_MIN_LEN;
+  if (max_q_len >= WA_MFMA_MIN_LEN) wa_prefill_launch(p, max_q_len, num_seqs, (hipStream_t)stream);
+  if (min_q_len < WA_MFMA_MIN_LEN) wa_decode_launch(p, num_tokens, (hipStream_t)stream);
+  APHRO_LAUNCH_CHECK();
+  return APHRO_OK;
+}

@@ -368,6 +368,43 @@ def windowed_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     return out
 
 
+def differential_window_attention_supported(heads: int, kv_heads: int, dim: int, vdim: int, dtype: torch.dtype) -> bool:
+    return dtype in _DT and bool(_lib.mixers_lib().aphro_differential_window_attention_supported(heads, kv_heads, dim, vdim, _DT[dtype]))
+
+
+def differential_window_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor,
+                                  v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                                  ctx_len: torch.Tensor, seq_of_token: torch.Tensor, q_len_range, heads: int, scale: float,
+                                  window: int, keep_first: int, lam: float, out_scale: float, eps: float) -> None:
+    """The two maps of every head under the window, joined (a_1 - lam a_2), unit RMS per head, out_scale, sigmoid gate, in one
+    launch: out [T, heads * vdim] (dense rows, any row stride).  Sizes as ``differential_window_attention_supported`` says."""
+    _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, q_len, ctx_len, seq_of_token)
+    lo, hi = int(q_len_range[0]), int(q_len_range[1])
+    _need(0 < lo <= hi, "differential_window_attention: q_len_range (shortest, longest)")
+    nb, bs, G2, d = k_cache.shape
+    G, e = v_cache.shape[2], v_cache.shape[3]
+    T, S = q.shape[0], q_start.numel()
+    _need(v_cache.shape[:2] == (nb, bs) and G2 == 2 * G and k_cache.is_contiguous() and v_cache.is_contiguous(),
+          "differential_window_attention: cache shapes")
+    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype and heads % G == 0 and out.shape == (T, heads * e),
+          "differential_window_attention: one dtype, out [T, heads * vdim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.is_contiguous(),
+          "differential_window_attention: block_tables int32 [S, max_blocks]")
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    _i32(seq_of_token, T, "seq_of_token")
+    gs = 0
+    if gate is not None:
+        _need(gate.dtype == q.dtype and gate.shape == (T, heads * e), "differential_window_attention: gate [T, heads * vdim]")
+        gs = _rows(gate, heads * e, "differential_window_attention gate")
+    check(_lib.mixers_lib().aphro_differential_window_attention(
+        out.data_ptr(), _rows(out, heads * e, "differential_window_attention out"), q.data_ptr(),
+        _rows(q, heads * 2 * d, "differential_window_attention q"), _p(gate), gs, k_cache.data_ptr(), v_cache.data_ptr(),
+        block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
+        seq_of_token.data_ptr(), T, S, lo, hi, heads, G, d, e, float(scale), int(window), int(keep_first), float(lam), float(out_scale),
+        float(eps), _dt(q), _stream()), "differential_window_attention")
+
+
 # ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------------
 def experts_route(router_out: torch.Tensor, correction: Optional[torch.Tensor], top: int):
     """router_out fp32 [T, outputs] -> (ids int32 [T, top], weights fp32 [T, top])."""

@@ -202,6 +202,13 @@ class WindowedMapsAttention(nn.Module):
         q = mops.short_conv(qkv, self.conv, conv_state, batch.state_slots, batch.q_start, batch.q_len, batch.ctx_len,
                             batch.seq_of_token, self.cq, self.ck, self.cv, k_cache if self.own_kv else None,
                             v_cache if self.own_kv else None, batch.slot_mapping if self.own_kv else None)
+        lens = (min(batch.q_lens), max(batch.q_lens))
+        if self.maps == 2 and mops.differential_window_attention_supported(self.heads, self.kv_heads, self.dim, self.vdim, q.dtype) \
+                and (gate is None or gate.stride(0) % 4 == 0):
+            mops.differential_window_attention(out, q, gate, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len,
+                                               batch.ctx_len, batch.seq_of_token, lens, self.heads, self.scale, self.window,
+                                               self.keep_first, self.lam, 1.0 - self.diff, self.eps)
+            return
         a = mops.windowed_attention(q, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len, batch.ctx_len,
                                     batch.seq_of_token, (min(batch.q_lens), max(batch.q_lens)), self.heads, self.maps, self.scale,
                                     self.window, self.keep_first,

@@ -147,6 +147,21 @@ int aphro_windowed_attention(float* out, int64_t out_stride, const void* q, int6
                              int heads, int kv_heads, int maps, int dim, int vdim, float scale, int window, int keep_first,
                              int max_kv_len, float* workspace, int64_t workspace_floats, int dtype, void* stream);
 
+/* Differential attention under the same window in one launch (bf16; dim, vdim in {32, 64, 96, 128}): the two maps of every head
+ * (q [T, heads * 2 * dim], k_cache [.., kv_heads * 2, dim], head by head as [map 1, map 2]) over the shared values,
+ *   o = a_1 - lambda * a_2;  out = out_scale * o / sqrt(mean(o^2) + eps) * sigmoid(gate)      (mean over the head's vdim values)
+ * out and gate [T, heads * vdim] of `dtype` (gate NULL: none).  Segments of 8 rows or more run on the matrix cores, shorter ones
+ * on the shared-key kernel.  aphro_differential_window_attention_supported says whether the sizes are served; what is not goes
+ * through aphro_windowed_attention and aphro_differential_norm_gate. */
+int aphro_differential_window_attention_supported(int heads, int kv_heads, int dim, int vdim, int dtype);
+int aphro_differential_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
+                                        int64_t gate_stride, const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                        int max_blocks, int64_t num_blocks, int block_size, const int32_t* q_start,
+                                        const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token,
+                                        int64_t num_tokens, int num_seqs, int min_q_len, int max_q_len, int heads, int kv_heads,
+                                        int dim, int vdim, float scale, int window, int keep_first, float lambda, float out_scale,
+                                        float eps, int dtype, void* stream);
+
 /* ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------
  * A SLOT is one (token, choice): slot = token * top + choice.
  * moe_route: router_out fp32 [T, outputs] -> ids int32 [T, top], weights fp32 [T, top]: s = softmax(router_out); the top

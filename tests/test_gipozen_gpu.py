@@ -256,6 +256,66 @@ def test_window_and_kept_tokens_end_exactly_where_they_should(mops, decoded, dty
             assert (col0 > 0.99).all() if seen else (col0 < 1e-6).all(), (row, key, seen, col0)
 
 
+FUSED_SHAPES = [  # heads, kv heads, dim, vdim, window, keep_first
+    (4, 1, 32, 96, 17, 3), (6, 2, 64, 32, 64, 0), (2, 2, 128, 128, 100, 1), (8, 2, 96, 64, 0, 0), (3, 3, 32, 32, 5, 70), (4, 2, 64, 128, 1, 0)]
+
+
+@pytest.mark.parametrize("shape", FUSED_SHAPES)
+def test_fused_differential_attention_in_mixed_batches(mops, shape):
+    """The one-launch form (both maps, join, unit RMS, gate) against the restatement: two sequences that advance together in
+    unequal segments -- portions of 8 rows and more beside shorter ones and single tokens -- over shuffled pages.  Every seventh
+    key is made loud, so a row that sees one key too many or too few at an edge of its window shows."""
+    H, G, d, e, window, keep = shape
+    assert mops.differential_window_attention_supported(H, G, d, e, torch.bfloat16)
+    rng = np.random.default_rng(H * d + e)
+    lens, block = (210, 77), 16
+    lam, diff, eps = 0.45, 0.3, 1e-5
+    seqs = []
+    for T in lens:
+        q = U.bf16_round(rng.standard_normal((T, H * 2 * d)))
+        k = rng.standard_normal((T, G * 2 * d))
+        k[3::7] *= 3.0
+        seqs.append((q, U.bf16_round(k), U.bf16_round(rng.standard_normal((T, G * e))), U.bf16_round(rng.standard_normal((T, H * e + 4)))))
+    want = [O.differential_attention(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), H, G, d, e, d ** -0.5,
+                                     window if window > 0 else 10 ** 6, keep, lam, diff, eps) * O.sigmoid(g[:, :H * e])
+            for q, k, v, g in seqs]
+    pages = [(T + block - 1) // block for T in lens]
+    perm = np.random.default_rng(2).permutation(sum(pages) + 2)
+    tables = [perm[:pages[0]], perm[pages[0]:pages[0] + pages[1]]]
+    bt = np.zeros((2, max(pages)), np.int32)
+    for i in range(2):
+        bt[i, :pages[i]] = tables[i]
+    kc = torch.full((sum(pages) + 2, block, G * 2, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((sum(pages) + 2, block, G, e), float("nan"), dtype=torch.bfloat16, device=DEV)
+    plan = [(70, 1), (2, 9), (1, 1), (64, 3), (9, 7), (1, 40), (63, 16)]
+    at, got = [0, 0], [[], []]
+    for step in plan:
+        live = [i for i in range(2) if step[i] and at[i] < lens[i]]
+        ns = [min(step[i], lens[i] - at[i]) for i in live]
+        order = sorted(range(len(live)), key=lambda j: ns[j] == 1 and at[live[j]] > 0)       # portions first, single tokens last
+        live, ns = [live[j] for j in order], [ns[j] for j in order]
+        starts = np.cumsum([0] + ns[:-1])
+        for i, n in zip(live, ns):
+            pos = np.arange(at[i], at[i] + n)
+            slots = torch.tensor(tables[i][pos // block] * block + pos % block, dtype=torch.int64, device=DEV)
+            kc.view(-1, G * 2 * d)[slots] = dev(seqs[i][1][at[i]:at[i] + n], torch.bfloat16)
+            vc.view(-1, G * e)[slots] = dev(seqs[i][2][at[i]:at[i] + n], torch.bfloat16)
+        q = dev(np.concatenate([seqs[i][0][at[i]:at[i] + n] for i, n in zip(live, ns)]), torch.bfloat16)
+        gate = dev(np.concatenate([seqs[i][3][at[i]:at[i] + n] for i, n in zip(live, ns)]), torch.bfloat16)
+        out = torch.zeros(q.shape[0], H * e + 8, dtype=torch.bfloat16, device=DEV)
+        mops.differential_window_attention(out[:, :H * e], q, gate[:, :H * e], kc, vc, torch.from_numpy(bt[live]).to(DEV).contiguous(),
+                                           i32(starts), i32(ns), i32([at[i] for i in live]),
+                                           i32(np.concatenate([[j] * n for j, n in enumerate(ns)])), (min(ns), max(ns)), H, d ** -0.5,
+                                           window, keep, lam, 1.0 - diff, eps)
+        assert float(out[:, H * e:].abs().max()) == 0.0
+        for j, (i, n) in enumerate(zip(live, ns)):
+            got[i].append(out[starts[j]:starts[j] + n, :H * e].float().cpu().numpy())
+            at[i] += n
+    for i in range(2):
+        assert at[i] == lens[i]
+        np.testing.assert_allclose(np.concatenate(got[i]), want[i], rtol=3e-2, atol=3e-2)
+
+
 def test_decoded_rows_far_past_the_window(mops):
     H, G, M, d, e = 4, 2, 2, 32, 64
     rng = np.random.default_rng(9)
