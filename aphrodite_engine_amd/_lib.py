@@ -183,12 +183,13 @@ MIXERS_SIGNATURES = {
     "aphro_windowed_attention": (I, [P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, I, F, I, I, I, P, L, I, P]),
     "aphro_differential_window_attention_supported": (I, [I, I, I, I, I]),
     "aphro_differential_window_attention": (I, [P, L, P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, F, I, I, F, F,
-                                            F, I, P]),
+                                            F, I, P, L, I, P]),
     "aphro_experts_route": (I, [P, P, P, P, L, I, I, P]),
     "aphro_experts_align_capacity": (L, [L, I]),
     "aphro_experts_align": (I, [P, L, P, P, P, L, I, P]),
-    "aphro_experts_glu_gemm": (I, [P, P, L, P, P, P, P, L, I, I, I, F, F, I, P]),
-    "aphro_experts_down_gemm": (I, [P, P, P, P, P, P, L, I, I, I, I, P]),
+    "aphro_experts_block_rows": (I, [L, I]),
+    "aphro_experts_glu_gemm": (I, [P, P, L, P, P, P, P, L, L, I, I, I, I, F, F, I, P]),
+    "aphro_experts_down_gemm": (I, [P, P, P, P, P, P, L, L, I, I, I, I, I, P]),
     "aphro_experts_combine": (I, [P, P, P, P, P, L, P, L, P, L, L, I, I, I, I, P]),
     "aphro_clamped_glu": (I, [P, P, L, L, I, F, F, I, P]),
 }

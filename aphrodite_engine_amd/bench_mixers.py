@@ -1,7 +1,10 @@
-"""``bench.py --mixers``: prefill and decode throughput of a Fatudra stack at sizes that resemble a real model's layers
+"""``bench.py --mixers [--mixers-design fatudra|gipozen]``: prefill and decode throughput of a Fatudra (or Gipozen) stack at sizes that resemble a real model's layers
 (random bf16 weights), beside a Llama stack of equal width / heads / feed-forward / layer count on the unquantised op path,
 plus each mixer kernel alone against its roofline and against the like kernel of the Llama path.  Prints ONE JSON line;
-the default workload of bench.py is untouched by it.
+the default workload of bench.py is untouched by it.  The Gipozen stack: windowed differential attention (two maps of half the
+head size over shared values, window 1024 + 4 kept tokens, 4-tap convolutions), every second layer reading the previous
+layer's keys and values and carrying 16 + 2 experts (top 4, a quarter of the dense feed-forward each, one shared expert)
+instead of the PolyNorm feed-forward; its expert products are priced against the MFMA figure over the ACTIVE experts' flops.
 
 Rooflines used: 8 TB/s HBM for the memory-bound kernels (norms, activations, decode attention, the decode step of the
 memories: their state is read and written once), 2.5 PFLOP/s dense bf16 MFMA for prompt attention (4 d flops per visible
@@ -36,6 +39,26 @@ def fatudra_config(s):
           "mlp": {"kind": "dense", "ff": s["ff"]}}
     return {"architecture": "Fatudra", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
             "layers": [par, ml, par, par][:LAYERS]}
+
+
+def gipozen_config(s):
+    d = s["dim"] // 2                       # two maps of half the head size: q is as wide as a plain head's
+    mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": s["dim"], "conv": 4, "diff": 0.3,
+             "mask": {"size": GIP_WINDOW, "keep_first": GIP_KEEP}, "scale": d ** -0.5}
+    eff = s["ff"] // 4 // 32 * 32
+    dense = {"kind": "dense", "ff": s["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0}, "router": {"experts": GIP_EXPERTS, "identity": 2, "top": GIP_TOP},
+           "shared": {"ff": eff, "limit": 7.0}}
+    layers = []
+    for i in range(LAYERS):
+        m = dict(mixer)
+        if i % 2:
+            m["kv_from"] = i - 1
+        layers.append({"type": "attention", "mixer": m, "mlp": moe if i % 2 else dense})
+    return {"architecture": "Gipozen", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0, "layers": layers}
+
+
+GIP_WINDOW, GIP_KEEP, GIP_EXPERTS, GIP_TOP = 1024, 4, 16, 4
 
 
 def timed(fn, iters=10, warmup=3):
@@ -164,8 +187,136 @@ def kernel_section(s, prompt_len, batch, ctx, device):
     return out
 
 
+def gipozen_kernel_section(s, prompt_len, batch, ctx, device):
+    """Each Gipozen kernel alone at the stack's shapes, and the like kernel of the Llama path at the same shapes."""
+    from . import _custom_ops as ops
+    from . import mixer_ops as mops
+    from .mixers import PagedKVSpec
+    bf = torch.bfloat16
+    H, G, e, W, ff = s["heads"], s["kv_heads"], s["dim"], s["width"], s["ff"]
+    d = e // 2
+    eff = ff // 4 // 32 * 32
+    pre, dec, pages = batches(prompt_len, batch, ctx, device, VOCAB)
+    out = {}
+
+    def rec(name, sec, bytes_=None, flops=None, like=None):
+        r = {"us": round(sec * 1e6, 1)}
+        if bytes_ is not None:
+            r["frac_hbm"] = round(bytes_ / sec / HBM, 3)
+        if flops is not None:
+            r["frac_mfma"] = round(flops / sec / MFMA, 4)
+        if like is not None:
+            r["like"] = like
+        out[name] = r
+
+    def visible_pairs(T):
+        return sum(min(i + 1, GIP_WINDOW) + min(GIP_KEEP, max(0, i + 1 - GIP_WINDOW)) for i in range(T))
+
+    # ---- attention: both maps, join, norm and gate in one launch ---------------------------------------------------------
+    kc, vc = PagedKVSpec(G, d, e, 2).allocate(pages, BLOCK, batch, bf, device)
+    kc.normal_()
+    vc.normal_()
+    for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+        q = torch.randn(T, H * 2 * d, device=device, dtype=bf)
+        gate = torch.randn(T, H * e, device=device, dtype=bf)
+        o = torch.empty(T, H * e, device=device, dtype=bf)
+        sec = timed(lambda: mops.differential_window_attention(o, q, gate, kc, vc, b.block_tables, b.q_start, b.q_len, b.ctx_len,
+                                                               b.seq_of_token, (min(b.q_lens), max(b.q_lens)), H, d ** -0.5, GIP_WINDOW,
+                                                               GIP_KEEP, 0.2, 0.7, 1e-6,
+                                                               max_kv_len=max(c + n for c, n in zip(b.ctx_lens, b.q_lens))))
+        if name == "prefill":
+            pairs = visible_pairs(T)
+            flops = pairs * H * (4.0 * d + 4.0 * e)              # two maps: Q K^T over d, P V over e, each twice
+            lq = torch.randn(T, H, e, device=device, dtype=bf)
+            k = torch.randn(T, G, e, device=device, dtype=bf)
+            v = torch.randn(T, G, e, device=device, dtype=bf)
+            cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+            lsec = timed(lambda: ops.flash_attn_varlen(lq, k, v, cu, T, e ** -0.5, causal=True, window_size=(GIP_WINDOW - 1, 0)))
+            lflops = pairs * H * 4.0 * e
+            rec("attention_prefill", sec, flops=flops, like={"kernel": "flash_attn_varlen (window)", "us": round(lsec * 1e6, 1),
+                                                             "frac_mfma": round(lflops / lsec / MFMA, 4)})
+        else:
+            nvis = min(ctx + 1, GIP_WINDOW) + min(GIP_KEEP, max(0, ctx + 1 - GIP_WINDOW))
+            nbytes = batch * nvis * G * (2 * d + e) * 2
+            lq = torch.randn(T, H, e, device=device, dtype=bf)
+            lk = torch.randn(pages, G, e // 8, BLOCK, 8, device=device, dtype=bf)
+            lv = torch.randn(pages, G, e, BLOCK, device=device, dtype=bf)
+            lens = torch.full((batch, ), ctx + 1, dtype=torch.int32, device=device)
+            lo = torch.empty(T, H, e, device=device, dtype=bf)
+            lsec = timed(lambda: ops.paged_attention_v1(lo, lq, lk, lv, G, e ** -0.5, b.block_tables, lens, BLOCK, ctx + 1, None,
+                                                        "auto", 1.0, 1.0))
+            lbytes = batch * (ctx + 1) * G * 2 * e * 2
+            rec("attention_decode", sec, bytes_=nbytes, like={"kernel": "paged_attention_v1", "us": round(lsec * 1e6, 1),
+                                                              "frac_hbm": round(lbytes / lsec / HBM, 3)})
+    # ---- convolution + cache write, norms, activation ---------------------------------------------------------------------
+    C = H * 2 * d + G * 2 * d + G * e
+    for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+        u = torch.randn(T, C + H * e, device=device, dtype=bf)
+        w = torch.randn(C, 4, device=device, dtype=bf)
+        state = torch.zeros(batch, 3, C, device=device, dtype=bf)
+        sec = timed(lambda: mops.short_conv(u[:, :C], w, state, b.state_slots, b.q_start, b.q_len, b.ctx_len, b.seq_of_token,
+                                            H * 2 * d, G * 2 * d, G * e, kc, vc, b.slot_mapping))
+        k = torch.randn(T, G, e, device=device, dtype=bf)
+        lkc = torch.zeros(pages, G, e // 8, BLOCK, 8, device=device, dtype=bf)
+        lvc = torch.zeros(pages, G, e, BLOCK, device=device, dtype=bf)
+        lq = torch.randn(T, H * e, device=device, dtype=bf)
+        lk = torch.randn(T, G * e, device=device, dtype=bf)
+        pos = b.positions
+        cs = torch.randn(8192, e, device=device, dtype=bf)
+        lsec = timed(lambda: (ops.rotary_embedding(pos, lq, lk, e, cs, True), ops.reshape_and_cache(k, k, lkc, lvc, b.slot_mapping, "auto", 1.0, 1.0)))
+        rec("short_conv_cache_" + name, sec, bytes_=T * C * 4,
+            like={"kernel": "rotary_embedding + reshape_and_cache", "us": round(lsec * 1e6, 1),
+                  "frac_hbm": round(T * (H + 3 * G) * e * 4 / lsec / HBM, 3)})
+        n_hist = LAYERS // 2
+        hist = torch.randn(LAYERS + 1, T, W, device=device)
+        x = torch.randn(T, W, device=device)
+        y = torch.randn(T, W, device=device, dtype=bf)
+        dw = torch.randn(n_hist + 1, device=device)
+        sec = timed(lambda: mops.depth_residual_rms_norm(x, x_out=x, y=y, history=hist, n_hist=n_hist, depth_w=dw, gain=1.1))
+        x16, r16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
+        w16 = torch.randn(W, device=device, dtype=bf)
+        lsec = timed(lambda: ops.fused_add_rms_norm(x16, r16, w16, 1e-5))
+        rec("depth_residual_rms_norm_" + name, sec, bytes_=T * W * (4 + 2 + 4 + 4 * n_hist + 4 + 2),
+            like={"kernel": "fused_add_rms_norm", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * W * 8 / lsec / HBM, 3)})
+        sec = timed(lambda: mops.depth_residual_rms_norm(x, x_out=x, y=y, gain=1.1))
+        rec("residual_rms_norm_" + name, sec, bytes_=T * W * (4 + 2 + 4 + 2))
+        z = torch.randn(T, ff, device=device, dtype=bf)
+        sec = timed(lambda: mops.poly_norm(z, (0.7, 0.5, 0.3, 0.1), 1e-6))
+        gu = torch.randn(T, 2 * ff, device=device, dtype=bf)
+        lo = torch.empty(T, ff, device=device, dtype=bf)
+        lsec = timed(lambda: ops.silu_and_mul(lo, gu))
+        rec("poly_norm_" + name, sec, bytes_=T * ff * 4,
+            like={"kernel": "silu_and_mul", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * ff * 6 / lsec / HBM, 3)})
+        # ---- experts: route, sort, both products, combine -- against the dense feed-forward's library products of equal active size
+        h = torch.randn(T, W, device=device, dtype=bf)
+        R = GIP_EXPERTS + 2
+        zr = torch.randn(T, R, device=device)
+        ids, wts = mops.experts_route(zr, None, GIP_TOP)
+        wgu = torch.randn(GIP_EXPERTS, 2 * eff, W, device=device, dtype=bf) * W ** -0.5
+        wdn = torch.randn(GIP_EXPERTS, W, eff, device=device, dtype=bf) * eff ** -0.5
+        sec = timed(lambda: mops.experts_forward(h, ids, wts, wgu, wdn, 7.0, 1.702))
+        wl1 = torch.randn(2 * GIP_TOP * eff, W, device=device, dtype=bf)
+        wl2 = torch.randn(W, GIP_TOP * eff, device=device, dtype=bf)
+        act = torch.randn(T, GIP_TOP * eff, device=device, dtype=bf)
+        lsec = timed(lambda: (torch.nn.functional.linear(h, wl1), torch.nn.functional.linear(act, wl2)))
+        flops = 6.0 * T * GIP_TOP * eff * W
+        wbytes = GIP_EXPERTS * 3 * eff * W * 2
+        r = {"kernel": "library products of the dense feed-forward at the active size", "us": round(lsec * 1e6, 1)}
+        if name == "prefill":
+            r["frac_mfma"] = round(flops / lsec / MFMA, 4)
+            rec("experts_" + name, sec, flops=flops, like=r)
+        else:
+            r["frac_hbm"] = round(3 * GIP_TOP * eff * W * 2 / lsec / HBM, 3)
+            rec("experts_" + name, sec, bytes_=wbytes, like=r)
+        sec = timed(lambda: mops.experts_route(zr, None, GIP_TOP))
+        rec("experts_route_" + name, sec)
+    return out
+
+
 def main(args) -> int:
     from . import _lib
+    if getattr(args, "mixers_design", "fatudra") == "gipozen":
+        return main_gipozen(args)
     from .fatudra import FatudraConfig, FatudraForCausalLM
     from .model import LlamaConfig, LlamaForCausalLM
     _lib.lib()
@@ -191,6 +342,40 @@ def main(args) -> int:
             r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
             del llama
             r["kernels"] = kernel_section(s, prompt_len, batch, ctx, device)
+            r["seconds"] = round(time.time() - t0, 1)
+            result["sizes"][name] = r
+            torch.cuda.empty_cache()
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def main_gipozen(args) -> int:
+    from . import _lib
+    from .gipozen import GipozenConfig, GipozenForCausalLM
+    from .model import LlamaConfig, LlamaForCausalLM
+    _lib.lib()
+    _lib.mixers_lib()
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    prompt_len, batch, ctx = args.mixers_prompt, args.batch, args.ctx
+    result = {"metric": "gipozen_vs_llama_bf16_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "n_gpus": 1, "layers": LAYERS, "sizes": {}}
+    with torch.no_grad():
+        for name, s in SIZES.items():
+            if args.mixers_size and name != args.mixers_size:
+                continue
+            t0 = time.time()
+            gip = GipozenForCausalLM(GipozenConfig.from_dict(gipozen_config(s)), torch.bfloat16).init_synthetic(device)
+            r = {"gipozen": model_throughput(gip, prompt_len, batch, ctx, device, VOCAB)}
+            del gip
+            lc = LlamaConfig(hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=LAYERS,
+                             num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=VOCAB,
+                             max_position_embeddings=max(8192, prompt_len + 16))
+            llama = LlamaForCausalLM(lc, None, torch.bfloat16).init_synthetic(device)
+            llama.use_fused_decode = False
+            r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
+            del llama
+            r["kernels"] = gipozen_kernel_section(s, prompt_len, batch, ctx, device)
             r["seconds"] = round(time.time() - t0, 1)
             result["sizes"][name] = r
             torch.cuda.empty_cache()

@@ -134,6 +134,27 @@ __global__ void depth_residual_rms_norm_vec8_kernel(const float* __restrict__ x_
   if (act) dn_store8<T>(out + at, r);
 }
 
+// three sums over a workgroup of up to 16 waves in one LDS round trip; red: >= 48 floats
+__device__ __forceinline__ void wg_sum3(float& a, float& b, float& c, float* red) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  c = wave_sum(c);
+  const int nw = (blockDim.x + 63) >> 6;
+  if (nw == 1) return;
+  if ((threadIdx.x & 63) == 0) {
+    red[3 * (threadIdx.x >> 6)] = a;
+    red[3 * (threadIdx.x >> 6) + 1] = b;
+    red[3 * (threadIdx.x >> 6) + 2] = c;
+  }
+  __syncthreads();
+  a = b = c = 0.f;
+  for (int w = 0; w < nw; ++w) {
+    a += red[3 * w];
+    b += red[3 * w + 1];
+    c += red[3 * w + 2];
+  }
+}
+
 template <typename T>
 __global__ void poly_norm_kernel(typename T::storage* __restrict__ out, const typename T::storage* __restrict__ z,
                                  int64_t z_stride, int n, float a, float b, float c, float e, float eps) {
@@ -163,7 +184,7 @@ __global__ void poly_norm_kernel(typename T::storage* __restrict__ out, const ty
 template <typename T>
 __global__ void poly_norm_vec8_kernel(typename T::storage* __restrict__ out, const typename T::storage* __restrict__ z,
                                       int64_t z_stride, int n, float a, float b, float c, float e, float eps) {
-  __shared__ float red[16];
+  __shared__ float red[48];
   const int64_t t = blockIdx.x;
   float v[2][8];
   bool act[2];
@@ -184,9 +205,10 @@ __global__ void poly_norm_vec8_kernel(typename T::storage* __restrict__ out, con
       s6 += v2 * v2 * v2;
     }
   const float inv = 1.0f / (float)n;
-  const float r1 = a / sqrtf(wg_sum(s2, red) * inv + eps);
-  const float r2 = b / sqrtf(wg_sum(s4, red) * inv + eps);
-  const float r3 = c / sqrtf(wg_sum(s6, red) * inv + eps);
+  wg_sum3(s2, s4, s6, red);
+  const float r1 = a / sqrtf(s2 * inv + eps);
+  const float r2 = b / sqrtf(s4 * inv + eps);
+  const float r3 = c / sqrtf(s6 * inv + eps);
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int i0 = (threadIdx.x + h * blockDim.x) * 8;

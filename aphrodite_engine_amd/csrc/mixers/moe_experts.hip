@@ -1,6 +1,7 @@
 // Mixture of small feed-forward experts on unquantised weights (bf16 on the matrix cores, fp32 on the vector ALUs):
 //   moe_route          softmax over the router's outputs, choice by score + correction, weight = the score itself
-//   moe_align          the (token, choice) slots sorted by expert into blocks of 16 rows, one expert per block
+//   moe_align          the (token, choice) slots sorted by expert into blocks of 16 (64, 128 in prompt-sized steps) rows, one
+//                      expert per block
 //   moe_glu_gemm       per block: [gate | up] product of its expert with the clamped gated activation in the epilogue
 //   moe_down_gemm      per block: the expert's down product, fp32 rows scattered back to their slots
 //   moe_combine        per token: weighted sum over its choices (identity experts pass the input through), plus the
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ id
 // one workgroup sorts every slot of the step
 __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ sorted_slots, int32_t* __restrict__ block_expert,
                                                          int32_t* __restrict__ num_blocks, const int32_t* __restrict__ ids,
-                                                         int64_t num_slots, int experts) {
+                                                         int64_t num_slots, int experts, int bm) {
   extern __shared__ int32_t li[];
   int32_t* count = li;
   int32_t* start = li + experts;
@@ -99,15 +100,15 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
     int off = 0;
     for (int e = 0; e < experts; ++e) {
       start[e] = off;
-      off += (count[e] + MOE_BM - 1) / MOE_BM * MOE_BM;
+      off += (count[e] + bm - 1) / bm * bm;
     }
     total = off;
-    num_blocks[0] = off / MOE_BM;
+    num_blocks[0] = off / bm;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < experts; e += blockDim.x) {
-    const int nb = (count[e] + MOE_BM - 1) / MOE_BM;
-    for (int j = 0; j < nb; ++j) block_expert[start[e] / MOE_BM + j] = e;
+    const int nb = (count[e] + bm - 1) / bm;
+    for (int j = 0; j < nb; ++j) block_expert[start[e] / bm + j] = e;
     count[e] = 0;                              // becomes the expert's cursor
   }
   for (int i = threadIdx.x; i < total; i += blockDim.x) sorted_slots[i] = -1;
@@ -118,54 +119,69 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
   }
 }
 
-// bf16 on v_mfma_f32_16x16x32_bf16: the weight rows are the A operand (16 output columns), the block's 16 rows the B operand,
-// so a lane ends with 4 consecutive output columns of one row.  One wave per 16 output columns, four waves per workgroup; both
-// operands come straight from global memory in 16-byte pieces along K (the block's rows are re-read by the four waves out of
-// the cache; the weights are read once per block).
-template <bool GLU>
+// bf16 on v_mfma_f32_16x16x32_bf16: the weight rows are the A operand (16 output columns), the block's rows the B operand, so
+// a lane ends with 4 consecutive output columns of one row.  A block is MT tiles of 16 rows; a wave owns all of them for 16
+// output columns of the gated product (gate and up rows: 2 MT products per 32 of K from MT + 2 operand loads) or 32 columns of
+// the down product, four waves per workgroup side by side along N.  Operands come straight from global memory in 16-byte
+// pieces along K: with MT = 4 or 8 (prompt-sized steps, where an expert has hundreds of rows) every weight piece feeds MT
+// products, with MT = 1 (decoded tokens: a handful of rows per expert) the weights are simply streamed once per block.
+template <bool GLU, int MT>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(void* __restrict__ out, const uint16_t* __restrict__ a, int64_t a_stride,
                                                             const uint16_t* __restrict__ w, const int32_t* __restrict__ sorted_slots,
                                                             const int32_t* __restrict__ block_expert,
                                                             const int32_t* __restrict__ num_blocks, int top, int N, int K,
                                                             float limit, float alpha) {
+  constexpr int BM = 16 * MT, NT = 2;                       // NT weight tiles per wave: (gate, up) of 16 columns, or 32 columns
   const int b = blockIdx.x;
   if (b >= num_blocks[0]) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  const int n0 = (blockIdx.y * 4 + wave) * (GLU ? 16 : 32);
   if (n0 >= N) return;
   const int e = block_expert[b];
-  const int slot = sorted_slots[b * MOE_BM + c];
-  const uint16_t* ar;
-  bool a_live = true;
-  if (GLU) {
-    a_live = slot >= 0;
-    ar = a + (int64_t)(a_live ? slot / top : 0) * a_stride + 8 * g;
-  } else {
-    ar = a + (int64_t)(b * MOE_BM + c) * a_stride + 8 * g;
+  int slot[MT];
+  const uint16_t* ar[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    slot[mt] = sorted_slots[b * BM + 16 * mt + c];
+    if (GLU) ar[mt] = a + (int64_t)(slot[mt] >= 0 ? slot[mt] / top : 0) * a_stride + 8 * g;
+    else ar[mt] = a + (int64_t)(b * BM + 16 * mt + c) * a_stride + 8 * g;
   }
+  const bool second = GLU || n0 + 16 < N;                   // the down product's second tile may lie beyond N
   const uint16_t* w0 = w + ((int64_t)e * (GLU ? 2 : 1) * N + n0 + c) * K + 8 * g;
-  const uint16_t* w1 = w0 + (int64_t)N * K;                 // GLU: the up rows
-  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-#pragma unroll 4
+  const uint16_t* w1 = GLU ? w0 + (int64_t)N * K : (second ? w0 + (int64_t)16 * K : w0);
+  f32x4 acc[NT][MT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
   for (int k0 = 0; k0 < K; k0 += 32) {
-    u32x4 af = *reinterpret_cast<const u32x4*>(ar + k0);
-    if (GLU && !a_live) af = zero;
     const u32x4 wf0 = *reinterpret_cast<const u32x4*>(w0 + k0);
-    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf0), __builtin_bit_cast(bf16x8, af), acc0, 0, 0, 0);
-    if (GLU) {
-      const u32x4 wf1 = *reinterpret_cast<const u32x4*>(w1 + k0);
-      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf1), __builtin_bit_cast(bf16x8, af), acc1, 0, 0, 0);
+    const u32x4 wf1 = *reinterpret_cast<const u32x4*>(w1 + k0);
+    u32x4 af[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) af[mt] = *reinterpret_cast<const u32x4*>(ar[mt] + k0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf0), __builtin_bit_cast(bf16x8, af[mt]),
+                                                           acc[0][mt], 0, 0, 0);
+      acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf1), __builtin_bit_cast(bf16x8, af[mt]),
+                                                           acc[1][mt], 0, 0, 0);
     }
   }
-  if (GLU) {
-    uint16_t* y = (uint16_t*)out + (int64_t)(b * MOE_BM + c) * N + n0 + 4 * g;
-    float v[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) v[r] = a_live ? clamped_glu_f(acc0[r], acc1[r], limit, alpha) : 0.f;
-    *reinterpret_cast<u32x2*>(y) = u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
-  } else if (slot >= 0) {
-    *reinterpret_cast<f32x4*>((float*)out + (int64_t)slot * N + n0 + 4 * g) = acc0;
+  for (int mt = 0; mt < MT; ++mt) {
+    if (GLU) {
+      uint16_t* y = (uint16_t*)out + (int64_t)(b * BM + 16 * mt + c) * N + n0 + 4 * g;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = slot[mt] >= 0 ? clamped_glu_f(acc[0][mt][r], acc[1][mt][r], limit, alpha) : 0.f;
+      *reinterpret_cast<u32x2*>(y) = u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
+    } else if (slot[mt] >= 0) {
+      float* d = (float*)out + (int64_t)slot[mt] * N + n0 + 4 * g;
+      *reinterpret_cast<f32x4*>(d) = acc[0][mt];
+      if (second) *reinterpret_cast<f32x4*>(d + 16) = acc[1][mt];
+    }
   }
 }
 
@@ -176,18 +192,18 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(void* __restrict__ 
                                                              const int32_t* __restrict__ sorted_slots,
                                                              const int32_t* __restrict__ block_expert,
                                                              const int32_t* __restrict__ num_blocks, int top, int N, int K,
-                                                             float limit, float alpha) {
-  const int b = blockIdx.x;
-  if (b >= num_blocks[0]) return;
-  const int m = threadIdx.x & 15, n = blockIdx.y * 16 + (threadIdx.x >> 4);
+                                                             float limit, float alpha, int bm) {
+  const int row = blockIdx.x * 16 + (threadIdx.x & 15);     // row of sorted_slots; a block of bm rows has one expert
+  if (row >= num_blocks[0] * bm) return;
+  const int n = blockIdx.y * 16 + (threadIdx.x >> 4);
   if (n >= N) return;
-  const int e = block_expert[b];
-  const int slot = sorted_slots[b * MOE_BM + m];
+  const int e = block_expert[row / bm];
+  const int slot = sorted_slots[row];
   if (slot < 0) {
-    if (GLU) ((typename T::storage*)out)[(int64_t)(b * MOE_BM + m) * N + n] = T::from_f32(0.f);
+    if (GLU) ((typename T::storage*)out)[(int64_t)row * N + n] = T::from_f32(0.f);
     return;
   }
-  const typename T::storage* ar = GLU ? a + (int64_t)(slot / top) * a_stride : a + (int64_t)(b * MOE_BM + m) * a_stride;
+  const typename T::storage* ar = GLU ? a + (int64_t)(slot / top) * a_stride : a + (int64_t)row * a_stride;
   const typename T::storage* w0 = w + ((int64_t)e * (GLU ? 2 : 1) * N + n) * K;
   const typename T::storage* w1 = w0 + (int64_t)N * K;
   float acc0 = 0.f, acc1 = 0.f;
@@ -196,7 +212,7 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(void* __restrict__ 
     acc0 += x * T::to_f32(w0[k]);
     if (GLU) acc1 += x * T::to_f32(w1[k]);
   }
-  if (GLU) ((typename T::storage*)out)[(int64_t)(b * MOE_BM + m) * N + n] = T::from_f32(clamped_glu_f(acc0, acc1, limit, alpha));
+  if (GLU) ((typename T::storage*)out)[(int64_t)row * N + n] = T::from_f32(clamped_glu_f(acc0, acc1, limit, alpha));
   else ((float*)out)[(int64_t)slot * N + n] = acc0;
 }
 
@@ -245,47 +261,71 @@ extern "C" int aphro_experts_route(int32_t* ids, float* weights, const float* ro
   return APHRO_OK;
 }
 
+// rows per block: 16 for a handful of rows per expert, 64 / 128 where an expert has hundreds (the prompt-sized products then
+// reuse every weight piece 4 / 8 times)
+extern "C" int aphro_experts_block_rows(int64_t num_slots, int experts) {
+  const int64_t per = num_slots / (experts > 0 ? experts : 1);
+  return per >= 512 ? 128 : (per >= 48 ? 64 : MOE_BM);
+}
+
 extern "C" int64_t aphro_experts_align_capacity(int64_t num_slots, int experts) {
-  return (num_slots + (int64_t)experts * (MOE_BM - 1) + MOE_BM - 1) / MOE_BM * MOE_BM;
+  const int bm = aphro_experts_block_rows(num_slots, experts);
+  return (num_slots + (int64_t)experts * (bm - 1) + bm - 1) / bm * bm;
 }
 
 extern "C" int aphro_experts_align(int32_t* sorted_slots, int64_t capacity, int32_t* block_expert, int32_t* num_blocks,
-                               const int32_t* ids, int64_t num_slots, int experts, void* stream) {
+                                   const int32_t* ids, int64_t num_slots, int experts, void* stream) {
   APHRO_CHECK(sorted_slots && block_expert && num_blocks && ids && num_slots > 0 && experts > 0 && experts <= 4096,
-              "moe_align: bad arguments (%d experts)", experts);
-  APHRO_CHECK(capacity >= aphro_experts_align_capacity(num_slots, experts) && capacity < 0x7fffffff, "moe_align: capacity too small");
+              "experts_align: bad arguments (%d experts)", experts);
+  APHRO_CHECK(capacity >= aphro_experts_align_capacity(num_slots, experts) && capacity < 0x7fffffff, "experts_align: capacity too small");
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * experts * sizeof(int32_t), (hipStream_t)stream,
-                     sorted_slots, block_expert, num_blocks, ids, num_slots, experts);
+                     sorted_slots, block_expert, num_blocks, ids, num_slots, experts, aphro_experts_block_rows(num_slots, experts));
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;
 }
 
+template <bool GLU>
+static void moe_gemm_bf16_launch(int bm, dim3 grid, hipStream_t st, void* out, const uint16_t* a, int64_t a_stride, const uint16_t* w,
+                                 const int32_t* sorted_slots, const int32_t* block_expert, const int32_t* num_blocks, int top, int N,
+                                 int K, float limit, float alpha) {
+  if (bm == 128)
+    hipLaunchKernelGGL((moe_gemm_bf16_kernel<GLU, 8>), grid, dim3(256), 0, st, out, a, a_stride, w, sorted_slots, block_expert,
+                       num_blocks, top, N, K, limit, alpha);
+  else if (bm == 64)
+    hipLaunchKernelGGL((moe_gemm_bf16_kernel<GLU, 4>), grid, dim3(256), 0, st, out, a, a_stride, w, sorted_slots, block_expert,
+                       num_blocks, top, N, K, limit, alpha);
+  else
+    hipLaunchKernelGGL((moe_gemm_bf16_kernel<GLU, 1>), grid, dim3(256), 0, st, out, a, a_stride, w, sorted_slots, block_expert,
+                       num_blocks, top, N, K, limit, alpha);
+}
+
 static int moe_gemm(bool glu, void* out, const void* a, int64_t a_stride, const void* w, const int32_t* sorted_slots,
-                    const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int N, int K, float limit,
-                    float alpha, int dtype, void* stream) {
-  APHRO_CHECK(out && a && w && sorted_slots && block_expert && num_blocks && capacity > 0 && capacity % MOE_BM == 0 && top > 0 &&
-                  N > 0 && K > 0 && a_stride >= K, "moe gemm: bad arguments");
-  const unsigned blocks = (unsigned)(capacity / MOE_BM);
+                    const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int64_t num_slots, int experts, int top,
+                    int N, int K, float limit, float alpha, int dtype, void* stream) {
+  const int bm = aphro_experts_block_rows(num_slots, experts);
+  APHRO_CHECK(out && a && w && sorted_slots && block_expert && num_blocks && capacity > 0 && capacity % bm == 0 && top > 0 &&
+                  N > 0 && K > 0 && a_stride >= K && capacity == aphro_experts_align_capacity(num_slots, experts),
+              "experts gemm: bad arguments");
   const bool mfma = dtype == APHRO_BF16 && N % 16 == 0 && K % 32 == 0 && a_stride % 8 == 0 && ((uintptr_t)a & 15) == 0 &&
                     ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0;
   if (mfma) {
-    const dim3 grid(blocks, (unsigned)((N + 63) / 64));
+    const dim3 grid((unsigned)(capacity / bm), (unsigned)((N + (glu ? 63 : 127)) / (glu ? 64 : 128)));
     if (glu)
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<true>), grid, dim3(256), 0, (hipStream_t)stream, out, (const uint16_t*)a, a_stride,
-                         (const uint16_t*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+      moe_gemm_bf16_launch<true>(bm, grid, (hipStream_t)stream, out, (const uint16_t*)a, a_stride, (const uint16_t*)w, sorted_slots,
+                                 block_expert, num_blocks, top, N, K, limit, alpha);
     else
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<false>), grid, dim3(256), 0, (hipStream_t)stream, out, (const uint16_t*)a, a_stride,
-                         (const uint16_t*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+      moe_gemm_bf16_launch<false>(bm, grid, (hipStream_t)stream, out, (const uint16_t*)a, a_stride, (const uint16_t*)w, sorted_slots,
+                                  block_expert, num_blocks, top, N, K, limit, alpha);
   } else {
-    const dim3 grid(blocks, (unsigned)((N + 15) / 16));
+    const dim3 grid((unsigned)(capacity / 16), (unsigned)((N + 15) / 16));
     MIX_DISPATCH_DTYPE(dtype, {
       typedef typename T::storage S;
       if (glu)
         hipLaunchKernelGGL((moe_gemm_plain_kernel<T, true>), grid, dim3(256), 0, (hipStream_t)stream, out, (const S*)a, a_stride,
-                           (const S*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+                           (const S*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha, bm);
       else
         hipLaunchKernelGGL((moe_gemm_plain_kernel<T, false>), grid, dim3(256), 0, (hipStream_t)stream, out, (const S*)a, a_stride,
-                           (const S*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+                           (const S*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha, bm);
     });
   }
   APHRO_LAUNCH_CHECK();
@@ -293,17 +333,17 @@ static int moe_gemm(bool glu, void* out, const void* a, int64_t a_stride, const 
 }
 
 extern "C" int aphro_experts_glu_gemm(void* y, const void* h, int64_t h_stride, const void* w_gate_up, const int32_t* sorted_slots,
-                                  const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int ff,
-                                  int width, float limit, float alpha, int dtype, void* stream) {
-  return moe_gemm(true, y, h, h_stride, w_gate_up, sorted_slots, block_expert, num_blocks, capacity, top, ff, width, limit, alpha,
-                  dtype, stream);
+                                  const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int64_t num_slots,
+                                  int experts, int top, int ff, int width, float limit, float alpha, int dtype, void* stream) {
+  return moe_gemm(true, y, h, h_stride, w_gate_up, sorted_slots, block_expert, num_blocks, capacity, num_slots, experts, top, ff,
+                  width, limit, alpha, dtype, stream);
 }
 
 extern "C" int aphro_experts_down_gemm(float* expert_out, const void* y, const void* w_down, const int32_t* sorted_slots,
-                                   const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int width,
-                                   int ff, int dtype, void* stream) {
-  return moe_gemm(false, expert_out, y, ff, w_down, sorted_slots, block_expert, num_blocks, capacity, top, width, ff, 0.f, 0.f,
-                  dtype, stream);
+                                   const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int64_t num_slots,
+                                   int experts, int top, int width, int ff, int dtype, void* stream) {
+  return moe_gemm(false, expert_out, y, ff, w_down, sorted_slots, block_expert, num_blocks, capacity, num_slots, experts, top, width,
+                  ff, 0.f, 0.f, dtype, stream);
 }
 
 extern "C" int aphro_experts_combine(void* out, const float* expert_out, const int32_t* ids, const float* weights, const void* h,

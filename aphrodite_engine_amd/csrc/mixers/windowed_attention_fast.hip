@@ -31,6 +31,8 @@ struct WAParams {
   int64_t out_stride, q_stride, gate_stride, num_blocks;
   int max_blocks, block_size, heads, kv_heads, dim, vdim, window, keep_first, min_len, bs_shift, max_tiles;
   float scale, lambda, out_scale, eps;
+  float* ws;                  // decoded rows, key range split over workgroups: partials [T, heads * 2, nsplit, 2 + vdim]
+  int nsplit;
 };
 
 __device__ __forceinline__ int wa_slot(const WAParams& p, const int32_t* bt, int key) {
@@ -321,7 +323,9 @@ __global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ck = lane & (CH - 1), kg = lane >> CHL;
   const bool kin = 8 * ck < p.dim, vin = 8 * ck < p.vdim;
-  const int head0 = kvh * (p.heads / p.kv_heads) + blockIdx.z * NHQ;
+  const int ngroups = p.heads / p.kv_heads / NHQ;
+  const int split = blockIdx.z / ngroups;
+  const int head0 = kvh * (p.heads / p.kv_heads) + (blockIdx.z % ngroups) * NHQ;
   float qv[QHM][8];
 #pragma unroll
   for (int qh = 0; qh < QHM; ++qh) {
@@ -341,7 +345,9 @@ __global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
     for (int j = 0; j < 8; ++j) acc[qh][j] = 0.f;
   }
   const int ntiles = (nvis + KT - 1) / KT;
-  for (int tile = wave; tile < ntiles; tile += 4) {
+  const int tps = (ntiles + p.nsplit - 1) / p.nsplit;
+  const int tile_end = min(ntiles, (split + 1) * tps);
+  for (int tile = split * tps + wave; tile < tile_end; tile += 4) {
     float sc[NI][QHM];
     u16x8 vv[NI];
 #pragma unroll
@@ -435,8 +441,18 @@ __global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
       L += merge[w][qh][1] * f;
       o += merge[w][qh][2 + col] * f;
     }
+    if (p.nsplit > 1) {                                     // this split's share; wa_merge_kernel finishes the row
+      float* w = p.ws + ((((int64_t)t * p.heads + head0) * 2 + qh) * p.nsplit + split) * (2 + p.vdim);
+      if (col == 0) {
+        w[0] = M;
+        w[1] = L;
+      }
+      w[2 + col] = o;
+      continue;
+    }
     fin[qh][col] = o / L;
   }
+  if (p.nsplit > 1) return;
   __syncthreads();
   if (wave >= NHQ) return;
   const int head = head0 + wave;
@@ -450,6 +466,51 @@ __global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
     float d = (fin[2 * wave][col] - p.lambda * fin[2 * wave + 1][col]) * rstd;
     if (p.gate) d *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head * p.vdim + col]));
     p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(d);
+  }
+}
+
+// one wave per (row, head): merges the key splits of both maps, joins, norms and gates.  vdim <= 256.
+__global__ __launch_bounds__(64) void wa_merge_kernel(WAParams p) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  if (p.q_len[p.seq_of_token[t]] >= p.min_len) return;
+  const int stride = 2 + p.vdim;
+  float a[2][4];
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp) {
+    const float* w = p.ws + (((int64_t)t * p.heads + head) * 2 + mp) * p.nsplit * stride;
+    float M = -INFINITY;
+    for (int z = 0; z < p.nsplit; ++z) M = fmaxf(M, w[z * stride]);
+    float L = 0.f;
+    for (int z = 0; z < p.nsplit; ++z) {
+      const float mz = w[z * stride];
+      if (mz != -INFINITY) L += w[z * stride + 1] * __expf(mz - M);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = lane + 64 * i;
+      float o = 0.f;
+      if (col < p.vdim)
+        for (int z = 0; z < p.nsplit; ++z) {
+          const float mz = w[z * stride];
+          if (mz != -INFINITY) o += w[z * stride + 2 + col] * __expf(mz - M);
+        }
+      a[mp][i] = o / L;
+    }
+  }
+  float d[4], ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    d[i] = a[0][i] - p.lambda * a[1][i];
+    ss += d[i] * d[i];
+  }
+  const float rstd = p.out_scale / sqrtf(wave_sum(ss) / (float)p.vdim + p.eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int col = lane + 64 * i;
+    if (col >= p.vdim) continue;
+    float v = d[i] * rstd;
+    if (p.gate) v *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head * p.vdim + col]));
+    p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(v);
   }
 }
 
@@ -498,7 +559,7 @@ static int wa_decode_qhm(int heads, int kv_heads, int dim, int vdim) {
 
 static void wa_decode_launch(const WAParams& p, int64_t num_tokens, hipStream_t st) {
   const int qhm = wa_decode_qhm(p.heads, p.kv_heads, p.dim, p.vdim), chl = wa_decode_chl(p.dim, p.vdim);
-  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)(p.heads / p.kv_heads / (qhm / 2)));
+  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)(p.heads / p.kv_heads / (qhm / 2) * p.nsplit));
 #define WDEC(QHM, CHL) hipLaunchKernelGGL((wa_decode_kernel<QHM, CHL>), grid, dim3(256), 0, st, p)
   if (qhm == 4) {
     switch (chl) {
@@ -515,6 +576,21 @@ static void wa_decode_launch(const WAParams& p, int64_t num_tokens, hipStream_t 
     }
   }
 #undef WDEC
+  if (p.nsplit > 1) hipLaunchKernelGGL(wa_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3(64), 0, st, p);
+}
+
+// Key splits of the decode kernel.  A decoded row is a chain of dependent loads (block table, then key and value rows) per step:
+// what shortens it is fewer steps per wave, so the splits go as far as one step per wave and sixteen workgroups per CU allow.
+static int wa_decode_splits(int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int max_visible, int64_t ws_floats) {
+  const int qhm = wa_decode_qhm(heads, kv_heads, dim, vdim), chl = wa_decode_chl(dim, vdim);
+  const int kt = 4 * (64 >> chl);
+  const int tiles = (max_visible + kt - 1) / kt;
+  const int64_t wgs = num_tokens * kv_heads * (heads / kv_heads / (qhm / 2));
+  int64_t n = (4096 + wgs - 1) / wgs;
+  if (n > tiles / 4) n = tiles / 4;
+  if (n > 8) n = 8;
+  while (n > 1 && num_tokens * heads * 2 * n * (2 + vdim) > ws_floats) --n;
+  return n < 1 ? 1 : (int)n;
 }
 
 constexpr int WA_MFMA_MIN_LEN = 8;
@@ -535,7 +611,8 @@ extern "C" int aphro_differential_window_attention(void* out, int64_t out_stride
                                                    const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
                                                    const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int min_q_len,
                                                    int max_q_len, int heads, int kv_heads, int dim, int vdim, float scale, int window,
-                                                   int keep_first, float lambda, float out_scale, float eps, int dtype, void* stream) {
+                                                   int keep_first, float lambda, float out_scale, float eps, int max_kv_len,
+                                                   float* workspace, int64_t workspace_floats, int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && q && k_cache && v_cache && block_tables && q_start && q_len && ctx_len && seq_of_token,
               "differential_window_attention: null argument");
@@ -561,6 +638,12 @@ extern "C" int aphro_differential_window_attention(void* out, int64_t out_stride
   for (int sft = 0; sft < 20; ++sft)
     if ((1 << sft) == block_size) p.bs_shift = sft;
   p.min_len = WA_MFMA_MIN_LEN;
+  p.ws = workspace;
+  p.nsplit = 1;
+  if (workspace && max_kv_len > 0) {
+    const int vis = window > 0 && window + keep_first < max_kv_len ? window + keep_first : max_kv_len;
+    p.nsplit = wa_decode_splits(num_tokens, heads, kv_heads, dim, vdim, vis, workspace_floats);
+  }
   if (max_q_len >= WA_MFMA_MIN_LEN) wa_prefill_launch(p, max_q_len, num_seqs, (hipStream_t)stream);
   if (min_q_len < WA_MFMA_MIN_LEN) wa_decode_launch(p, num_tokens, (hipStream_t)stream);
   APHRO_LAUNCH_CHECK();

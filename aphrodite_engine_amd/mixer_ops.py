@@ -375,9 +375,12 @@ def differential_window_attention_supported(heads: int, kv_heads: int, dim: int,
 def differential_window_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor,
                                   v_cache: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                                   ctx_len: torch.Tensor, seq_of_token: torch.Tensor, q_len_range, heads: int, scale: float,
-                                  window: int, keep_first: int, lam: float, out_scale: float, eps: float) -> None:
+                                  window: int, keep_first: int, lam: float, out_scale: float, eps: float,
+                                  max_kv_len: int = 0) -> None:
     """The two maps of every head under the window, joined (a_1 - lam a_2), unit RMS per head, out_scale, sigmoid gate, in one
-    launch: out [T, heads * vdim] (dense rows, any row stride).  Sizes as ``differential_window_attention_supported`` says."""
+    launch: out [T, heads * vdim] (dense rows, any row stride).  Sizes as ``differential_window_attention_supported`` says.
+    ``max_kv_len``: the longest ctx_len + q_len of the batch (host); given, decoded rows that see many keys split them over
+    several workgroups through a scratch tensor."""
     _cuda(out, q, gate, k_cache, v_cache, block_tables, q_start, q_len, ctx_len, seq_of_token)
     lo, hi = int(q_len_range[0]), int(q_len_range[1])
     _need(0 < lo <= hi, "differential_window_attention: q_len_range (shortest, longest)")
@@ -397,12 +400,17 @@ def differential_window_attention(out: torch.Tensor, q: torch.Tensor, gate: Opti
     if gate is not None:
         _need(gate.dtype == q.dtype and gate.shape == (T, heads * e), "differential_window_attention: gate [T, heads * vdim]")
         gs = _rows(gate, heads * e, "differential_window_attention gate")
+    ws, ws_n = None, 0
+    visible = min(max_kv_len, window + keep_first) if window > 0 else max_kv_len
+    if visible >= 512 and lo < 8:
+        ws_n = T * heads * 2 * 8 * (2 + e)
+        ws = torch.empty(ws_n, dtype=torch.float32, device=q.device)
     check(_lib.mixers_lib().aphro_differential_window_attention(
         out.data_ptr(), _rows(out, heads * e, "differential_window_attention out"), q.data_ptr(),
         _rows(q, heads * 2 * d, "differential_window_attention q"), _p(gate), gs, k_cache.data_ptr(), v_cache.data_ptr(),
         block_tables.data_ptr(), block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         seq_of_token.data_ptr(), T, S, lo, hi, heads, G, d, e, float(scale), int(window), int(keep_first), float(lam), float(out_scale),
-        float(eps), _dt(q), _stream()), "differential_window_attention")
+        float(eps), int(max_kv_len), _p(ws), ws_n, _dt(q), _stream()), "differential_window_attention")
 
 
 # ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------------
@@ -439,7 +447,7 @@ def experts_forward(h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w
     cap = int(lib.aphro_experts_align_capacity(T * top, E))
     dev = h.device
     sorted_slots = torch.empty(cap, dtype=torch.int32, device=dev)
-    block_expert = torch.empty(cap // 16, dtype=torch.int32, device=dev)
+    block_expert = torch.empty(cap // int(lib.aphro_experts_block_rows(T * top, E)), dtype=torch.int32, device=dev)
     num_blocks = torch.empty(1, dtype=torch.int32, device=dev)
     y = torch.empty(cap, ff, dtype=h.dtype, device=dev)
     eo = torch.empty(T * top, W, dtype=torch.float32, device=dev)
@@ -448,10 +456,10 @@ def experts_forward(h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w
     check(lib.aphro_experts_align(sorted_slots.data_ptr(), cap, block_expert.data_ptr(), num_blocks.data_ptr(), ids.data_ptr(),
                                   T * top, E, st), "experts_align")
     check(lib.aphro_experts_glu_gemm(y.data_ptr(), h.data_ptr(), hs, w_gate_up.data_ptr(), sorted_slots.data_ptr(),
-                                     block_expert.data_ptr(), num_blocks.data_ptr(), cap, top, ff, W, float(limit), float(alpha),
-                                     _dt(h), st), "experts_glu_gemm")
+                                     block_expert.data_ptr(), num_blocks.data_ptr(), cap, T * top, E, top, ff, W, float(limit),
+                                     float(alpha), _dt(h), st), "experts_glu_gemm")
     check(lib.aphro_experts_down_gemm(eo.data_ptr(), y.data_ptr(), w_down.data_ptr(), sorted_slots.data_ptr(),
-                                      block_expert.data_ptr(), num_blocks.data_ptr(), cap, top, W, ff, _dt(h), st),
+                                      block_expert.data_ptr(), num_blocks.data_ptr(), cap, T * top, E, top, W, ff, _dt(h), st),
           "experts_down_gemm")
     ss = sgs = 0
     if shared is not None:

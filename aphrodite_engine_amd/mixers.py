@@ -207,7 +207,8 @@ class WindowedMapsAttention(nn.Module):
                 and (gate is None or gate.stride(0) % 4 == 0):
             mops.differential_window_attention(out, q, gate, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len,
                                                batch.ctx_len, batch.seq_of_token, lens, self.heads, self.scale, self.window,
-                                               self.keep_first, self.lam, 1.0 - self.diff, self.eps)
+                                               self.keep_first, self.lam, 1.0 - self.diff, self.eps,
+                                               max_kv_len=max(c + n for c, n in zip(batch.ctx_lens, batch.q_lens)))
             return
         a = mops.windowed_attention(q, k_cache, v_cache, batch.block_tables, batch.q_start, batch.q_len, batch.ctx_len,
                                     batch.seq_of_token, (min(batch.q_lens), max(batch.q_lens)), self.heads, self.maps, self.scale,

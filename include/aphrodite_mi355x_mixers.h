@@ -151,7 +151,9 @@ int aphro_windowed_attention(float* out, int64_t out_stride, const void* q, int6
  * (q [T, heads * 2 * dim], k_cache [.., kv_heads * 2, dim], head by head as [map 1, map 2]) over the shared values,
  *   o = a_1 - lambda * a_2;  out = out_scale * o / sqrt(mean(o^2) + eps) * sigmoid(gate)      (mean over the head's vdim values)
  * out and gate [T, heads * vdim] of `dtype` (gate NULL: none).  Segments of 8 rows or more run on the matrix cores, shorter ones
- * on the shared-key kernel.  aphro_differential_window_attention_supported says whether the sizes are served; what is not goes
+ * on the shared-key kernel, which splits long key ranges over up to 8 workgroups per row when max_kv_len (host-side longest
+ * ctx_len + q_len) and an fp32 workspace of num_tokens * heads * 2 * splits * (2 + vdim) floats are given (NULL: no split).
+ * aphro_differential_window_attention_supported says whether the sizes are served; what is not goes
  * through aphro_windowed_attention and aphro_differential_norm_gate. */
 int aphro_differential_window_attention_supported(int heads, int kv_heads, int dim, int vdim, int dtype);
 int aphro_differential_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
@@ -160,7 +162,8 @@ int aphro_differential_window_attention(void* out, int64_t out_stride, const voi
                                         const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token,
                                         int64_t num_tokens, int num_seqs, int min_q_len, int max_q_len, int heads, int kv_heads,
                                         int dim, int vdim, float scale, int window, int keep_first, float lambda, float out_scale,
-                                        float eps, int dtype, void* stream);
+                                        float eps, int max_kv_len, float* workspace, int64_t workspace_floats, int dtype,
+                                        void* stream);
 
 /* ---- mixture of experts on unquantised weights ---------------------------------------------------------------------------
  * A SLOT is one (token, choice): slot = token * top + choice.
@@ -168,22 +171,24 @@ int aphro_differential_window_attention(void* out, int64_t out_stride, const voi
  *   values of s + correction (fp32 [outputs], NULL: none; ties to the lower index) are chosen, weights are their s. */
 int aphro_experts_route(int32_t* ids, float* weights, const float* router_out, const float* correction, int64_t num_tokens,
                     int outputs, int top, void* stream);
-/* rows of sorted_slots that any step of num_slots slots over `experts` experts can need (a multiple of 16) */
+/* rows per block of a step of num_slots slots over `experts` experts: 16, or 64 / 128 where an expert has hundreds of rows */
+int aphro_experts_block_rows(int64_t num_slots, int experts);
+/* rows of sorted_slots that such a step can need (a multiple of the block) */
 int64_t aphro_experts_align_capacity(int64_t num_slots, int experts);
-/* Sorts the slots whose id is below `experts` by expert into blocks of 16 rows (one expert per block, -1 pads a block):
- * sorted_slots int32 [capacity], block_expert int32 [capacity / 16], num_blocks int32 [1].  Other ids are left out. */
+/* Sorts the slots whose id is below `experts` by expert into blocks (one expert per block, -1 pads a block):
+ * sorted_slots int32 [capacity], block_expert int32 [capacity / block rows], num_blocks int32 [1].  Other ids are left out. */
 int aphro_experts_align(int32_t* sorted_slots, int64_t capacity, int32_t* block_expert, int32_t* num_blocks, const int32_t* ids,
                     int64_t num_slots, int experts, void* stream);
 /* y[row, :] of `dtype` [capacity, ff], row = place in sorted_slots: g = min(W_gate h, limit), u = clamp(W_up h, +-limit),
  * y = g * sigmoid(alpha * g) * (u + 1) with the block's expert; w_gate_up [experts, 2 * ff, width] (gate rows, then up rows);
  * h [T, width] (row stride), the slot's token is slot / top.  Rows of padding are zero. */
 int aphro_experts_glu_gemm(void* y, const void* h, int64_t h_stride, const void* w_gate_up, const int32_t* sorted_slots,
-                       const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int ff, int width,
-                       float limit, float alpha, int dtype, void* stream);
+                       const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int64_t num_slots, int experts,
+                       int top, int ff, int width, float limit, float alpha, int dtype, void* stream);
 /* expert_out fp32 [slots, width]: row slot = W_down(expert) y[its sorted row]; w_down [experts, width, ff]. */
 int aphro_experts_down_gemm(float* expert_out, const void* y, const void* w_down, const int32_t* sorted_slots,
-                        const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int top, int width, int ff,
-                        int dtype, void* stream);
+                        const int32_t* block_expert, const int32_t* num_blocks, int64_t capacity, int64_t num_slots, int experts,
+                        int top, int width, int ff, int dtype, void* stream);
 /* out[t] = sum_k weights[t, k] * (ids[t, k] < experts ? expert_out[t * top + k] : h[t])
  *          + sigmoid(shared_gate[t]) * shared[t]        (shared NULL: none; shared_gate NULL: ungated; one number per row) */
 int aphro_experts_combine(void* out, const float* expert_out, const int32_t* ids, const float* weights, const void* h,

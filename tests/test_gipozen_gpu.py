@@ -123,7 +123,7 @@ def conv_in_steps(mops, us, w, cuts, dtype, cq, ck, cv, slots=None, state=None, 
         lens = [len(r) for r in rows]
         starts = np.cumsum([0] + lens[:-1])
         u = dev(np.concatenate(rows), dtype)
-        pad = torch.zeros(u.shape[0], C + 8, dtype=dtype, device=DEV)
+        pad = torch.zeros(u.shape[0], C + 8, dtype=dtype, device=DEV)      # rows with a stride of their own
         pad[:, :C] = u
         seq_of = np.concatenate([[j] * n_ for j, n_ in enumerate(lens)])
         slot_map = torch.tensor(np.concatenate([base[i] + at[i] + np.arange(n_) for i, n_ in zip(live, lens)]), dtype=torch.int64,
@@ -145,9 +145,10 @@ def conv_in_steps(mops, us, w, cuts, dtype, cq, ck, cv, slots=None, state=None, 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 3, 4, 7])
-def test_short_conv_in_steps_of_every_size(mops, dtype, taps):
+@pytest.mark.parametrize("channels", [(52, 20, 37), (48, 16, 40)])      # the second: rows that are read 16 bytes at a time
+def test_short_conv_in_steps_of_every_size(mops, dtype, taps, channels):
     rng = np.random.default_rng(taps)
-    cq, ck, cv = 52, 20, 37
+    cq, ck, cv = channels
     C = cq + ck + cv
     w = rounded(rng.standard_normal((C, taps)), dtype)
     us = [rounded(rng.standard_normal((n, C)), dtype) for n in (29, 1, 12)]
@@ -314,6 +315,42 @@ def test_fused_differential_attention_in_mixed_batches(mops, shape):
     for i in range(2):
         assert at[i] == lens[i]
         np.testing.assert_allclose(np.concatenate(got[i]), want[i], rtol=3e-2, atol=3e-2)
+
+
+def test_fused_decoded_rows_split_long_key_ranges(mops):
+    """Decoded rows that see a thousand keys: their key range is cut over several workgroups and merged."""
+    H, G, d, e, window, keep = 4, 2, 64, 128, 1000, 3
+    lam, diff, eps = 0.3, 0.25, 1e-5
+    rng = np.random.default_rng(11)
+    T, block = 1300, 16
+    q = U.bf16_round(rng.standard_normal((T, H * 2 * d)))
+    k = U.bf16_round(rng.standard_normal((T, G * 2 * d)))
+    v = U.bf16_round(rng.standard_normal((T, G * e)))
+    pages = (T + block - 1) // block
+    perm = np.random.default_rng(2).permutation(pages)
+    pos = np.arange(T)
+    slots = torch.tensor(perm[pos // block] * block + pos % block, dtype=torch.int64, device=DEV)
+    kc = torch.zeros(pages, block, G * 2, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(pages, block, G, e, dtype=torch.bfloat16, device=DEV)
+    kc.view(-1, G * 2 * d)[slots] = dev(k, torch.bfloat16)
+    vc.view(-1, G * e)[slots] = dev(v, torch.bfloat16)
+    rows = [1290, 1295, 1299]
+    qq, kk, vv = q.reshape(T, H, 2, d), k.reshape(T, G, 2, d), v.reshape(T, G, e)
+    for row in rows:
+        out = torch.zeros(1, H * e, dtype=torch.bfloat16, device=DEV)
+        mops.differential_window_attention(out, dev(q[row:row + 1], torch.bfloat16), None, kc, vc, i32(perm).view(1, -1), i32([0]), i32([1]),
+                                           i32([row]), i32([0]), (1, 1), H, d ** -0.5, window, keep, lam, 1.0 - diff, eps, max_kv_len=row + 1)
+        js = [j for j in range(row + 1) if O.visible(row, j, window, keep)]
+        assert len(js) == window + keep
+        want = np.zeros((H, e))
+        for h in range(H):
+            a = []
+            for m in range(2):
+                sc = kk[js, h // 2, m] @ qq[row, h, m] * d ** -0.5
+                pr = np.exp(sc - sc.max())
+                a.append((pr / pr.sum()) @ vv[js, h // 2])
+            want[h] = O.rms_unit(a[0] - lam * a[1], eps) * (1.0 - diff)
+        np.testing.assert_allclose(out.float().cpu().numpy().reshape(H, e), want, rtol=3e-2, atol=3e-2)
 
 
 def test_decoded_rows_far_past_the_window(mops):
