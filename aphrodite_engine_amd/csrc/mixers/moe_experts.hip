@@ -185,6 +185,122 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(void* __restrict__ o
   }
 }
 
+// Prompt-sized steps, blocks of 128 rows: a workgroup owns the block's 128 rows x 128 weight rows (the gated product: 64 output
+// columns, their gate rows and their up rows; the down product: 128 columns) and walks K in steps of 64: both tiles go through
+// LDS (16-byte chunks XOR-swizzled by row so that the 16 rows of a fragment read hit different banks), the next step's pieces are
+// in flight in registers while the current step's 32 products per wave run.  Waves 2 x 2: 64 rows x 64 weight rows each.
+constexpr int TG_BM = 128, TG_BN = 128, TG_BK = 64;
+
+template <bool GLU>
+__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(void* __restrict__ out, const uint16_t* __restrict__ a, int64_t a_stride,
+                                                             const uint16_t* __restrict__ w, const int32_t* __restrict__ sorted_slots,
+                                                             const int32_t* __restrict__ block_expert,
+                                                             const int32_t* __restrict__ num_blocks, int top, int N, int K,
+                                                             float limit, float alpha) {
+  __shared__ __attribute__((aligned(16))) uint16_t a_lds[TG_BM * TG_BK];
+  __shared__ __attribute__((aligned(16))) uint16_t w_lds[TG_BN * TG_BK];
+  __shared__ int32_t slot_lds[TG_BM];
+  const int b = blockIdx.x;
+  if (b >= num_blocks[0]) return;
+  const int e = block_expert[b];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int ncols = GLU ? TG_BN / 2 : TG_BN;               // output columns of the workgroup
+  const int n0 = blockIdx.y * ncols;
+  if (threadIdx.x < TG_BM) slot_lds[threadIdx.x] = sorted_slots[b * TG_BM + threadIdx.x];
+  // this thread's pieces of the two tiles: 4 + 4 chunks of 16 bytes per K step
+  const uint16_t* ap[4];
+  const uint16_t* wp[4];
+  int lds_at[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = threadIdx.x + 256 * i, row = idx >> 3, ch = idx & 7;
+    lds_at[i] = row * TG_BK + 8 * (ch ^ (row & 7));
+    if (GLU) {
+      const int slot = sorted_slots[b * TG_BM + row];
+      ap[i] = a + (int64_t)(slot >= 0 ? slot / top : 0) * a_stride + 8 * ch;
+      const int col = min(n0 + (row & 63), N - 1);          // weight rows 0..63: gate, 64..127: up, of the same columns
+      wp[i] = w + ((int64_t)e * 2 * N + (row < 64 ? 0 : N) + col) * K + 8 * ch;
+    } else {
+      ap[i] = a + (int64_t)(b * TG_BM + row) * a_stride + 8 * ch;
+      wp[i] = w + ((int64_t)e * N + min(n0 + row, N - 1)) * K + 8 * ch;
+    }
+  }
+  f32x4 acc[4][4];                                          // [row tile][weight tile]
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  u32x4 ra[4], rw[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    ra[i] = *reinterpret_cast<const u32x4*>(ap[i]);
+    rw[i] = *reinterpret_cast<const u32x4*>(wp[i]);
+  }
+  for (int k0 = 0; k0 < K; k0 += TG_BK) {
+    __syncthreads();                                        // the previous step is consumed
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4*>(&a_lds[lds_at[i]]) = ra[i];
+      *reinterpret_cast<u32x4*>(&w_lds[lds_at[i]]) = rw[i];
+    }
+    __syncthreads();
+    if (k0 + TG_BK < K) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ra[i] = *reinterpret_cast<const u32x4*>(ap[i] + k0 + TG_BK);
+        rw[i] = *reinterpret_cast<const u32x4*>(wp[i] + k0 + TG_BK);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      u32x4 af[4], wf[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        const int row = 64 * wm + 16 * mt + c;
+        af[mt] = *reinterpret_cast<const u32x4*>(&a_lds[row * TG_BK + 8 * ((4 * ks + g) ^ (row & 7))]);
+      }
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        // the gated product: weight tiles {2 wn, 2 wn + 1} are gate rows, {4 + 2 wn, 5 + 2 wn} the up rows of the same columns
+        const int tile = GLU ? ((nt >> 1) * 4 + 2 * wn + (nt & 1)) : 4 * wn + nt;
+        const int row = 16 * tile + c;
+        wf[nt] = *reinterpret_cast<const u32x4*>(&w_lds[row * TG_BK + 8 * ((4 * ks + g) ^ (row & 7))]);
+      }
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[nt]), __builtin_bit_cast(bf16x8, af[mt]),
+                                                                acc[mt][nt], 0, 0, 0);
+    }
+  }
+  // a lane holds, per (row tile, weight tile), 4 consecutive weight rows 4 g .. 4 g + 3 of block row 64 wm + 16 mt + c
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int row = 64 * wm + 16 * mt + c;
+    const int slot = slot_lds[row];
+    if (GLU) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + 32 * wn + 16 * j + 4 * g;
+        if (col >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = slot >= 0 ? clamped_glu_f(acc[mt][j][r], acc[mt][2 + j][r], limit, alpha) : 0.f;
+        *reinterpret_cast<u32x2*>((uint16_t*)out + (int64_t)(b * TG_BM + row) * N + col) =
+            u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
+      }
+    } else if (slot >= 0) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int col = n0 + 64 * wn + 16 * nt + 4 * g;
+        if (col < N) *reinterpret_cast<f32x4*>((float*)out + (int64_t)slot * N + col) = acc[mt][nt];
+      }
+    }
+  }
+}
+
 // any storage type and size: thread = one output element of the block, fp32 multiply-adds along K
 template <typename T, bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(void* __restrict__ out, const typename T::storage* __restrict__ a,
@@ -308,7 +424,15 @@ static int moe_gemm(bool glu, void* out, const void* a, int64_t a_stride, const 
               "experts gemm: bad arguments");
   const bool mfma = dtype == APHRO_BF16 && N % 16 == 0 && K % 32 == 0 && a_stride % 8 == 0 && ((uintptr_t)a & 15) == 0 &&
                     ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0;
-  if (mfma) {
+  if (mfma && bm == TG_BM && K % TG_BK == 0 && N % 4 == 0) {
+    const dim3 grid((unsigned)(capacity / bm), (unsigned)((N + (glu ? 63 : 127)) / (glu ? 64 : 128)));
+    if (glu)
+      hipLaunchKernelGGL((moe_gemm_tiled_kernel<true>), grid, dim3(256), 0, (hipStream_t)stream, out, (const uint16_t*)a, a_stride,
+                         (const uint16_t*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+    else
+      hipLaunchKernelGGL((moe_gemm_tiled_kernel<false>), grid, dim3(256), 0, (hipStream_t)stream, out, (const uint16_t*)a, a_stride,
+                         (const uint16_t*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
+  } else if (mfma) {
     const dim3 grid((unsigned)(capacity / bm), (unsigned)((N + (glu ? 63 : 127)) / (glu ? 64 : 128)));
     if (glu)
       moe_gemm_bf16_launch<true>(bm, grid, (hipStream_t)stream, out, (const uint16_t*)a, a_stride, (const uint16_t*)w, sorted_slots,

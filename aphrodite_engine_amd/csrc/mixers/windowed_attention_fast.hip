@@ -9,10 +9,11 @@
 //    fragments read from LDS feed both maps.  Only key tiles that some row of the workgroup can see are visited: the tiles of the
 //    kept first tokens, then from the tile of the lowest window start on; a wave skips tiles none of its 16 rows sees, and the
 //    mask is applied only on tiles that are not wholly visible to the wave.
-//  * wa_decode_kernel<QHM, CHL>: the other rows (single decoded tokens, short portions), one workgroup per (row, kv head, group
-//    of QHM / 2 query heads): one pass over the row's visible keys -- numbered kept tokens first, then the window -- with a key
-//    row read by 2^CHL lanes x 16 bytes, partial dot products folded with DPP moves, each value row used by all QHM (head, map)
-//    pairs; four waves take the steps round-robin and merge through LDS, where the maps are then joined, normed and gated.
+//  * wa_decode_mfma_kernel<DK, DV>: the other rows (single decoded tokens, short portions), one workgroup per (row, kv head):
+//    the columns of a score tile are the kv head's query heads, the keys are the row's visible ones -- numbered kept tokens
+//    first, then the window -- staged through LDS like a prompt tile; long key ranges are split over workgroups and merged
+//    (wa_merge_kernel).  Measured before it: the same rows on the vector ALUs (a key row over 16 lanes, DPP-folded dot products)
+//    took 2 to 2.4 times as long at 1028 visible keys -- instruction-bound, whatever the split.
 #include "mixers_common.h"
 
 namespace aphro {
@@ -31,7 +32,7 @@ struct WAParams {
   int64_t out_stride, q_stride, gate_stride, num_blocks;
   int max_blocks, block_size, heads, kv_heads, dim, vdim, window, keep_first, min_len, bs_shift, max_tiles;
   float scale, lambda, out_scale, eps;
-  float* ws;                  // decoded rows, key range split over workgroups: partials [T, heads * 2, nsplit, 2 + vdim]
+  float* ws;                  // decoded rows, key range split over workgroups: partials [T, heads, 2 maps, nsplit, 2 + vdim]
   int nsplit;
 };
 
@@ -57,8 +58,11 @@ struct WAStage {
   u16x8 k[2][KI], v0[VI], v1[VI];
 };
 
+// Rows t0 .. t0 + 63 of a key numbering in which number r stands for key r below ns and for key lo + (r - ns) from there on
+// (a prompt tile passes ns = INT_MAX: the numbering is the keys themselves); nk: numbers in all.
 template <int DK, int DV>
-__device__ __forceinline__ void wa_load(WAStage<DK, DV>& st, const WAParams& p, const int32_t* bt, int kvh, int t0, int nk) {
+__device__ __forceinline__ void wa_load(WAStage<DK, DV>& st, const WAParams& p, const int32_t* bt, int kvh, int t0, int nk,
+                                        int ns = 0x7fffffff, int lo = 0) {
   constexpr int NCHK = DK / 8, NCHV = DV / 8;
   const int64_t krow = (int64_t)p.kv_heads * 2 * DK, vrow = (int64_t)p.kv_heads * DV;
 #pragma unroll
@@ -66,7 +70,8 @@ __device__ __forceinline__ void wa_load(WAStage<DK, DV>& st, const WAParams& p, 
     const int i = threadIdx.x + 256 * it;
     if (i < WA_BN * NCHK) {
       const int tok = i / NCHK, ch = i % NCHK;
-      const uint16_t* kr = p.k_cache + (int64_t)wa_slot(p, bt, min(t0 + tok, nk - 1)) * krow + (int64_t)kvh * 2 * DK + 8 * ch;
+      const int r = min(t0 + tok, nk - 1);
+      const uint16_t* kr = p.k_cache + (int64_t)wa_slot(p, bt, r < ns ? r : lo + (r - ns)) * krow + (int64_t)kvh * 2 * DK + 8 * ch;
       st.k[0][it] = *reinterpret_cast<const u16x8*>(kr);
       st.k[1][it] = *reinterpret_cast<const u16x8*>(kr + DK);
     }
@@ -78,7 +83,8 @@ __device__ __forceinline__ void wa_load(WAStage<DK, DV>& st, const WAParams& p, 
       const int tp = i / NCHV, ch = i % NCHV;
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const int key = min(t0 + 2 * tp + half, nk - 1);
+        const int r = min(t0 + 2 * tp + half, nk - 1);
+        const int key = r < ns ? r : lo + (r - ns);
         u16x8 vv = *reinterpret_cast<const u16x8*>(p.v_cache + (int64_t)wa_slot(p, bt, key) * vrow + kvh * DV + 8 * ch);
         if (t0 + 2 * tp + half >= nk) vv = u16x8{0, 0, 0, 0, 0, 0, 0, 0};    // beyond the sequence: no NaN into P V
         if (half == 0) st.v0[it] = vv;
@@ -303,174 +309,190 @@ __global__ __launch_bounds__(256) void wa_prefill_kernel(WAParams p) {
   }
 }
 
-// QHM (head, map) pairs = QHM / 2 query heads of one kv head per workgroup
-template <int QHM, int CHL>
-__global__ __launch_bounds__(256) void wa_decode_kernel(WAParams p) {
-  constexpr int CH = 1 << CHL;       // lanes per key row (16 bytes each)
-  constexpr int KP = 64 / CH;        // keys per load instruction
-  constexpr int NI = 4;              // load instructions per step of the online softmax
-  constexpr int KT = NI * KP;        // keys per step
-  constexpr int NHQ = QHM / 2;       // query heads of the workgroup
-  __shared__ float merge[4][QHM][2 + 8 * CH];
-  __shared__ float fin[QHM][8 * CH];
-  const int t = blockIdx.x, kvh = blockIdx.y;
+// Decoded rows on the matrix cores: a workgroup owns one row and one kv head; the 16 columns of a score tile are the kv head's
+// query heads (up to 16), so the two maps' keys and the shared values of a 64-key tile -- staged in LDS exactly as for a prompt
+// portion, over the row's visible keys numbered kept tokens first -- serve all of them.  The four waves divide a tile's work
+// by map and by half: wave 2 m + h takes map m and keys 32 h .. 32 h + 31, keeps its own running maximum, sum and output, and
+// the halves, then the maps, meet in LDS at the end (or, when the key range is split over workgroups, in wa_merge_kernel).
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void wa_decode_mfma_kernel(WAParams p) {
+  constexpr int NCHK = DK / 8, NKS = DK / 32, NDT = DV / 16;
+  constexpr int SWZ = (NCHK & -NCHK) - 1;
+  constexpr int KBYTES = 2 * WA_BN * DK * 2, VBYTES = DV * WA_VT * 2, MROW = DV + 2;
+  static_assert(KBYTES + VBYTES >= 2 * 16 * MROW * 4, "the merge buffer reuses the tiles' memory");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[KBYTES + VBYTES];
+  uint16_t* k_lds = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* vt_lds = reinterpret_cast<uint16_t*>(smem + KBYTES);
+  float* mrg = reinterpret_cast<float*>(smem);             // [2 maps][16 heads][2 + DV], after the last tile
+  const int t = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int seq = p.seq_of_token[t];
   if (p.q_len[seq] >= p.min_len) return;                   // the prompt kernel's share
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  const int mp = wave >> 1, pk = wave & 1;
+  const int QH = p.heads / p.kv_heads;
   const int pos = p.ctx_len[seq] + (t - p.q_start[seq]);
   const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
   const int ns = min(p.keep_first, lo);
   const int nvis = ns + pos - lo + 1;                      // visible keys: [0, ns) and [lo, pos]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int ck = lane & (CH - 1), kg = lane >> CHL;
-  const bool kin = 8 * ck < p.dim, vin = 8 * ck < p.vdim;
-  const int ngroups = p.heads / p.kv_heads / NHQ;
-  const int split = blockIdx.z / ngroups;
-  const int head0 = kvh * (p.heads / p.kv_heads) + (blockIdx.z % ngroups) * NHQ;
-  float qv[QHM][8];
+  constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+  const float qs = p.scale * LOG2E;
+  const int head = kvh * QH + min(c, QH - 1);              // columns beyond the kv head's query heads repeat the last one
+  u32x4 qf[NKS];
+  {
+    const uint16_t* qp = p.q + (int64_t)t * p.q_stride + ((int64_t)head * 2 + mp) * DK;
 #pragma unroll
-  for (int qh = 0; qh < QHM; ++qh) {
-    u16x8 raw = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    if (kin) raw = *reinterpret_cast<const u16x8*>(p.q + (int64_t)t * p.q_stride + ((int64_t)head0 * 2 + qh) * p.dim + 8 * ck);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) qv[qh][j] = BFloat::to_f32(raw[j]);
+    for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const u32x4*>(qp + 32 * ks + 8 * g);
   }
+  f32x4 o[NDT];
+#pragma unroll
+  for (int i = 0; i < NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
-  const int64_t krow = (int64_t)p.kv_heads * 2 * p.dim, vrow = (int64_t)p.kv_heads * p.vdim;
-  float m[QHM], l[QHM], acc[QHM][8];
-#pragma unroll
-  for (int qh = 0; qh < QHM; ++qh) {
-    m[qh] = -INFINITY;
-    l[qh] = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[qh][j] = 0.f;
-  }
-  const int ntiles = (nvis + KT - 1) / KT;
+  const int ntiles = (nvis + WA_BN - 1) / WA_BN;
   const int tps = (ntiles + p.nsplit - 1) / p.nsplit;
-  const int tile_end = min(ntiles, (split + 1) * tps);
-  for (int tile = split * tps + wave; tile < tile_end; tile += 4) {
-    float sc[NI][QHM];
-    u16x8 vv[NI];
+  const int r_end = min(ntiles, (split + 1) * tps) * WA_BN;
+  int r0 = split * tps * WA_BN;
+  WAStage<DK, DV> st;
+  if (r0 < r_end) wa_load<DK, DV>(st, p, bt, kvh, r0, nvis, ns, lo);
+  for (; r0 < r_end; r0 += WA_BN) {
+    __syncthreads();                                        // the previous tile is consumed
+    wa_store<DK, DV>(st, k_lds, vt_lds);
+    __syncthreads();
+    if (r0 + WA_BN < r_end) wa_load<DK, DV>(st, p, bt, kvh, r0 + WA_BN, nvis, ns, lo);
+    f32x4 s[2];
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int r = tile * KT + i * KP + kg;
-      const bool valid = r < nvis;
-      const int key = valid ? (r < ns ? r : lo + (r - ns)) : 0;
-      const int64_t slot = wa_slot(p, bt, key);
-      u16x8 k0 = u16x8{0, 0, 0, 0, 0, 0, 0, 0}, k1 = k0;
-      vv[i] = k0;
-      if (valid && kin) {
-        const uint16_t* kr = p.k_cache + slot * krow + (int64_t)kvh * 2 * p.dim + 8 * ck;
-        k0 = *reinterpret_cast<const u16x8*>(kr);
-        k1 = *reinterpret_cast<const u16x8*>(kr + p.dim);
-      }
-      if (valid && vin) vv[i] = *reinterpret_cast<const u16x8*>(p.v_cache + slot * vrow + kvh * p.vdim + 8 * ck);
-      float kf[2][8];
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int tok = 16 * (2 * pk + h2) + c;
+      s[h2] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        kf[0][j] = BFloat::to_f32(k0[j]);
-        kf[1][j] = BFloat::to_f32(k1[j]);
-      }
-#pragma unroll
-      for (int qh = 0; qh < QHM; ++qh) {
-        float d = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) d += qv[qh][j] * kf[qh & 1][j];
-        d = group_sum<CHL>(d);
-        sc[i][qh] = valid ? d * p.scale : -INFINITY;
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int ch = (4 * ks + g) ^ (tok & SWZ);
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(&k_lds[mp * WA_BN * DK + tok * DK + 8 * ch]);
+        s[h2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h2], 0, 0, 0);
       }
     }
+    float pv[2][4];
+    float mx = -INFINITY;
 #pragma unroll
-    for (int qh = 0; qh < QHM; ++qh) {
-      float mx = sc[0][qh];
+    for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-      for (int i = 1; i < NI; ++i) mx = fmaxf(mx, sc[i][qh]);
-#pragma unroll
-      for (int o = CH; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      const float m_new = fmaxf(m[qh], mx);                // finite: the tile's first key exists
-      const float alpha = (m[qh] == -INFINITY) ? 0.f : __expf(m[qh] - m_new);
-      m[qh] = m_new;
-      float ls = 0.f;
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const float e = (sc[i][qh] == -INFINITY) ? 0.f : __expf(sc[i][qh] - m_new);
-        sc[i][qh] = e;
-        ls += e;
+      for (int r = 0; r < 4; ++r) {
+        const int idx = r0 + 16 * (2 * pk + h2) + 4 * g + r;
+        const float xv = idx < nvis ? s[h2][r] * qs : -INFINITY;
+        pv[h2][r] = xv;
+        mx = fmaxf(mx, xv);
       }
-      l[qh] = l[qh] * alpha + ls;
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    m_run = m_new;
+    float lsum = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[qh][j] *= alpha;
-    }
+    for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float vf = BFloat::to_f32(vv[i][j]);
-#pragma unroll
-        for (int qh = 0; qh < QHM; ++qh) acc[qh][j] += sc[i][qh] * vf;
+      for (int r = 0; r < 4; ++r) {
+        const float e = __builtin_amdgcn_exp2f(pv[h2][r] - m_safe);
+        pv[h2][r] = e;
+        lsum += e;
       }
+    l_run = l_run * alpha + lsum;
+    const u32x4 pf = {pack2_16<true>(pv[0][0], pv[0][1]), pack2_16<true>(pv[0][2], pv[0][3]), pack2_16<true>(pv[1][0], pv[1][1]),
+                      pack2_16<true>(pv[1][2], pv[1][3])};
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      o[dt] *= alpha;
+      const uint16_t* vr = &vt_lds[(16 * dt + c) * WA_VT + 32 * pk + 4 * g];
+      const u32x2 vlo = *reinterpret_cast<const u32x2*>(vr);
+      const u32x2 vhi = *reinterpret_cast<const u32x2*>(vr + 16);
+      const u32x4 vf = {vlo[0], vlo[1], vhi[0], vhi[1]};
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
     }
   }
-  // fold the key groups of the wave, then the four waves
-#pragma unroll
-  for (int qh = 0; qh < QHM; ++qh) {
-#pragma unroll
-    for (int o = CH; o < 64; o <<= 1) {
-      l[qh] += __shfl_xor(l[qh], o, 64);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[qh][j] += __shfl_xor(acc[qh][j], o, 64);
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  __syncthreads();                                          // the tiles' memory becomes the merge buffer
+  float* mine = mrg + (mp * 16 + c) * MROW;
+  if (pk == 1) {                                            // the second half of the keys hands over to the first
+    if (g == 0) {
+      mine[0] = m_run;
+      mine[1] = l_run;
     }
-    if (lane == 0) {
-      merge[wave][qh][0] = m[qh];
-      merge[wave][qh][1] = l[qh];
-    }
-    if (kg == 0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) merge[wave][qh][2 + 8 * ck + j] = acc[qh][j];
-    }
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mine[2 + 16 * dt + 4 * g + r] = o[dt][r];
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < QHM * p.vdim; idx += 256) {
-    const int qh = idx / p.vdim, col = idx % p.vdim;
-    float M = -INFINITY;
+  if (pk == 0) {
+    const float m2 = mine[0], l2 = mine[1];
+    const float M = fmaxf(m_run, m2);
+    const float Ms = M == -INFINITY ? 0.f : M;
+    const float f1 = __builtin_amdgcn_exp2f(m_run - Ms), f2 = __builtin_amdgcn_exp2f(m2 - Ms);
+    l_run = l_run * f1 + l2 * f2;
+    m_run = M;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, merge[w][qh][0]);
-    float L = 0.f, o = 0.f;
+    for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float f = (merge[w][qh][0] == -INFINITY) ? 0.f : __expf(merge[w][qh][0] - M);
-      L += merge[w][qh][1] * f;
-      o += merge[w][qh][2 + col] * f;
-    }
-    if (p.nsplit > 1) {                                     // this split's share; wa_merge_kernel finishes the row
-      float* w = p.ws + ((((int64_t)t * p.heads + head0) * 2 + qh) * p.nsplit + split) * (2 + p.vdim);
-      if (col == 0) {
-        w[0] = M;
-        w[1] = L;
-      }
-      w[2 + col] = o;
-      continue;
-    }
-    fin[qh][col] = o / L;
+      for (int r = 0; r < 4; ++r) o[dt][r] = o[dt][r] * f1 + mine[2 + 16 * dt + 4 * g + r] * f2;
   }
-  if (p.nsplit > 1) return;
+  if (p.nsplit > 1) {                                       // this split's share of (head, map); wa_merge_kernel finishes the row
+    if (pk == 0 && c < QH) {
+      float* w = p.ws + ((((int64_t)t * p.heads + head) * 2 + mp) * p.nsplit + split) * (2 + DV);
+      if (g == 0) {
+        w[0] = m_run * LN2;                                 // wa_merge_kernel weighs with natural exponentials
+        w[1] = l_run;
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(w + 2 + 16 * dt + 4 * g) = o[dt];
+    }
+    return;
+  }
+  __syncthreads();                                          // map 1's first half has read what it was handed
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (wave == 2) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mine[2 + 16 * dt + 4 * g + r] = o[dt][r] * inv;
+  }
   __syncthreads();
-  if (wave >= NHQ) return;
-  const int head = head0 + wave;
+  if (wave != 0) return;
+  const float* a2 = mrg + (16 + c) * MROW + 2;
   float ss = 0.f;
-  for (int col = lane; col < p.vdim; col += 64) {
-    const float d = fin[2 * wave][col] - p.lambda * fin[2 * wave + 1][col];
-    ss += d * d;
-  }
-  const float rstd = p.out_scale / sqrtf(wave_sum(ss) / (float)p.vdim + p.eps);
-  for (int col = lane; col < p.vdim; col += 64) {
-    float d = (fin[2 * wave][col] - p.lambda * fin[2 * wave + 1][col]) * rstd;
-    if (p.gate) d *= sigmoid_f(BFloat::to_f32(p.gate[(int64_t)t * p.gate_stride + head * p.vdim + col]));
-    p.out[(int64_t)t * p.out_stride + head * p.vdim + col] = BFloat::from_f32(d);
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float d = o[dt][r] * inv - p.lambda * a2[16 * dt + 4 * g + r];
+      o[dt][r] = d;
+      ss += d * d;
+    }
+  ss += __shfl_xor(ss, 16, 64);
+  ss += __shfl_xor(ss, 32, 64);
+  if (c >= QH) return;
+  const float rstd = p.out_scale / sqrtf(ss / (float)DV + p.eps);
+  uint16_t* op = p.out + (int64_t)t * p.out_stride + head * DV + 4 * g;
+  const uint16_t* gp = p.gate ? p.gate + (int64_t)t * p.gate_stride + head * DV + 4 * g : nullptr;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = o[dt][r] * rstd;
+    if (gp) {
+      const u16x4 gg = *reinterpret_cast<const u16x4*>(gp + 16 * dt);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] *= sigmoid_f(BFloat::to_f32(gg[r]));
+    }
+    *reinterpret_cast<u32x2*>(op + 16 * dt) = u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
   }
 }
 
-// one wave per (row, head): merges the key splits of both maps, joins, norms and gates.  vdim <= 256.
+// one wave per (row, head): merges the key splits (at most 8) of both maps, joins, norms and gates.  vdim <= 256.  Every load
+// of a map is requested before the first is used.
 __global__ __launch_bounds__(64) void wa_merge_kernel(WAParams p) {
+  constexpr int MAXS = 8;
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   if (p.q_len[p.seq_of_token[t]] >= p.min_len) return;
   const int stride = 2 + p.vdim;
@@ -478,24 +500,28 @@ __global__ __launch_bounds__(64) void wa_merge_kernel(WAParams p) {
 #pragma unroll
   for (int mp = 0; mp < 2; ++mp) {
     const float* w = p.ws + (((int64_t)t * p.heads + head) * 2 + mp) * p.nsplit * stride;
+    float mz[MAXS], lz[MAXS], oz[MAXS][4];
+#pragma unroll
+    for (int z = 0; z < MAXS; ++z) {
+      const bool on = z < p.nsplit;
+      mz[z] = on ? w[z * stride] : -INFINITY;
+      lz[z] = on ? w[z * stride + 1] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) oz[z][i] = (on && lane + 64 * i < p.vdim) ? w[z * stride + 2 + lane + 64 * i] : 0.f;
+    }
     float M = -INFINITY;
-    for (int z = 0; z < p.nsplit; ++z) M = fmaxf(M, w[z * stride]);
-    float L = 0.f;
-    for (int z = 0; z < p.nsplit; ++z) {
-      const float mz = w[z * stride];
-      if (mz != -INFINITY) L += w[z * stride + 1] * __expf(mz - M);
+#pragma unroll
+    for (int z = 0; z < MAXS; ++z) M = fmaxf(M, mz[z]);
+    float L = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int z = 0; z < MAXS; ++z) {
+      const float f = mz[z] == -INFINITY ? 0.f : __expf(mz[z] - M);
+      L += lz[z] * f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] += oz[z][i] * f;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int col = lane + 64 * i;
-      float o = 0.f;
-      if (col < p.vdim)
-        for (int z = 0; z < p.nsplit; ++z) {
-          const float mz = w[z * stride];
-          if (mz != -INFINITY) o += w[z * stride + 2 + col] * __expf(mz - M);
-        }
-      a[mp][i] = o / L;
-    }
+    for (int i = 0; i < 4; ++i) a[mp][i] = o[i] / L;
   }
   float d[4], ss = 0.f;
 #pragma unroll
@@ -542,52 +568,38 @@ static void wa_prefill_launch(const WAParams& p0, int max_q_len, int num_seqs, h
   }
 }
 
-static int wa_decode_chl(int dim, int vdim) {
-  const int pieces = (max(dim, vdim) + 7) / 8;
-  int chl = 2;
-  while ((1 << chl) < pieces) ++chl;
-  return chl;
-}
-
-// (head, map) pairs per workgroup: 4 where the kv head has an even number of query heads and the row fits, else 2
-static int wa_decode_qhm(int heads, int kv_heads, int dim, int vdim) {
-  const int chl = wa_decode_chl(dim, vdim);
-  if ((dim & 7) || (vdim & 7) || chl > 5) return 0;
-  if ((heads / kv_heads) % 2 == 0 && 4 * (1 << chl) <= 64) return 4;
-  return 2;
-}
-
-static void wa_decode_launch(const WAParams& p, int64_t num_tokens, hipStream_t st) {
-  const int qhm = wa_decode_qhm(p.heads, p.kv_heads, p.dim, p.vdim), chl = wa_decode_chl(p.dim, p.vdim);
-  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)(p.heads / p.kv_heads / (qhm / 2) * p.nsplit));
-#define WDEC(QHM, CHL) hipLaunchKernelGGL((wa_decode_kernel<QHM, CHL>), grid, dim3(256), 0, st, p)
-  if (qhm == 4) {
-    switch (chl) {
-      case 2: WDEC(4, 2); break;
-      case 3: WDEC(4, 3); break;
-      case 4: WDEC(4, 4); break;
-    }
-  } else {
-    switch (chl) {
-      case 2: WDEC(2, 2); break;
-      case 3: WDEC(2, 3); break;
-      case 4: WDEC(2, 4); break;
-      case 5: WDEC(2, 5); break;
-    }
+template <int DK>
+static void wa_launch_decode_mfma_dv(const WAParams& p, dim3 grid, hipStream_t st) {
+  switch (p.vdim) {
+    case 32: hipLaunchKernelGGL((wa_decode_mfma_kernel<DK, 32>), grid, dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((wa_decode_mfma_kernel<DK, 64>), grid, dim3(256), 0, st, p); break;
+    case 96: hipLaunchKernelGGL((wa_decode_mfma_kernel<DK, 96>), grid, dim3(256), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((wa_decode_mfma_kernel<DK, 128>), grid, dim3(256), 0, st, p); break;
   }
-#undef WDEC
+}
+
+// decoded rows on the matrix cores: kv heads of up to 16 query heads, the prompt kernel's sizes
+static bool wa_decode_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
+  return wa_prefill_supported(dim, vdim) && heads / kv_heads <= 16 && vdim % 4 == 0;
+}
+
+static void wa_decode_mfma_launch(const WAParams& p, int64_t num_tokens, hipStream_t st) {
+  const dim3 grid((unsigned)num_tokens, (unsigned)p.kv_heads, (unsigned)p.nsplit);
+  switch (p.dim) {
+    case 32: wa_launch_decode_mfma_dv<32>(p, grid, st); break;
+    case 64: wa_launch_decode_mfma_dv<64>(p, grid, st); break;
+    case 96: wa_launch_decode_mfma_dv<96>(p, grid, st); break;
+    case 128: wa_launch_decode_mfma_dv<128>(p, grid, st); break;
+  }
   if (p.nsplit > 1) hipLaunchKernelGGL(wa_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3(64), 0, st, p);
 }
 
-// Key splits of the decode kernel.  A decoded row is a chain of dependent loads (block table, then key and value rows) per step:
-// what shortens it is fewer steps per wave, so the splits go as far as one step per wave and sixteen workgroups per CU allow.
-static int wa_decode_splits(int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int max_visible, int64_t ws_floats) {
-  const int qhm = wa_decode_qhm(heads, kv_heads, dim, vdim), chl = wa_decode_chl(dim, vdim);
-  const int kt = 4 * (64 >> chl);
-  const int tiles = (max_visible + kt - 1) / kt;
-  const int64_t wgs = num_tokens * kv_heads * (heads / kv_heads / (qhm / 2));
-  int64_t n = (4096 + wgs - 1) / wgs;
-  if (n > tiles / 4) n = tiles / 4;
+// key splits of the matrix-core decode kernel: a thousand workgroups, at least two tiles each
+static int wa_decode_mfma_splits(int64_t num_tokens, int heads, int kv_heads, int vdim, int max_visible, int64_t ws_floats) {
+  const int tiles = (max_visible + WA_BN - 1) / WA_BN;
+  const int64_t wgs = num_tokens * kv_heads;
+  int64_t n = (1024 + wgs - 1) / wgs;
+  if (n > tiles / 2) n = tiles / 2;
   if (n > 8) n = 8;
   while (n > 1 && num_tokens * heads * 2 * n * (2 + vdim) > ws_floats) --n;
   return n < 1 ? 1 : (int)n;
@@ -602,7 +614,7 @@ using namespace aphro;
 /* 1 if aphro_differential_window_attention serves these sizes (bf16 only), else 0 */
 extern "C" int aphro_differential_window_attention_supported(int heads, int kv_heads, int dim, int vdim, int dtype) {
   if (dtype != APHRO_BF16 || heads <= 0 || kv_heads <= 0 || heads % kv_heads) return 0;
-  return wa_decode_qhm(heads, kv_heads, dim, vdim) != 0 && wa_prefill_supported(dim, vdim) ? 1 : 0;
+  return wa_decode_mfma_supported(heads, kv_heads, dim, vdim) ? 1 : 0;
 }
 
 extern "C" int aphro_differential_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
@@ -642,10 +654,10 @@ extern "C" int aphro_differential_window_attention(void* out, int64_t out_stride
   p.nsplit = 1;
   if (workspace && max_kv_len > 0) {
     const int vis = window > 0 && window + keep_first < max_kv_len ? window + keep_first : max_kv_len;
-    p.nsplit = wa_decode_splits(num_tokens, heads, kv_heads, dim, vdim, vis, workspace_floats);
+    p.nsplit = wa_decode_mfma_splits(num_tokens, heads, kv_heads, vdim, vis, workspace_floats);
   }
   if (max_q_len >= WA_MFMA_MIN_LEN) wa_prefill_launch(p, max_q_len, num_seqs, (hipStream_t)stream);
-  if (min_q_len < WA_MFMA_MIN_LEN) wa_decode_launch(p, num_tokens, (hipStream_t)stream);
+  if (min_q_len < WA_MFMA_MIN_LEN) wa_decode_mfma_launch(p, num_tokens, (hipStream_t)stream);
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;
 }

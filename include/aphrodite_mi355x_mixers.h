@@ -150,8 +150,8 @@ int aphro_windowed_attention(float* out, int64_t out_stride, const void* q, int6
 /* Differential attention under the same window in one launch (bf16; dim, vdim in {32, 64, 96, 128}): the two maps of every head
  * (q [T, heads * 2 * dim], k_cache [.., kv_heads * 2, dim], head by head as [map 1, map 2]) over the shared values,
  *   o = a_1 - lambda * a_2;  out = out_scale * o / sqrt(mean(o^2) + eps) * sigmoid(gate)      (mean over the head's vdim values)
- * out and gate [T, heads * vdim] of `dtype` (gate NULL: none).  Segments of 8 rows or more run on the matrix cores, shorter ones
- * on the shared-key kernel, which splits long key ranges over up to 8 workgroups per row when max_kv_len (host-side longest
+ * out and gate [T, heads * vdim] of `dtype` (gate NULL: none); at most 16 query heads per kv head.  Segments of 8 rows or more
+ * run on the prompt kernel, shorter ones on the decode kernel (a kv head's query heads side by side), which splits long key ranges over up to 8 workgroups per row when max_kv_len (host-side longest
  * ctx_len + q_len) and an fp32 workspace of num_tokens * heads * 2 * splits * (2 + vdim) floats are given (NULL: no split).
  * aphro_differential_window_attention_supported says whether the sizes are served; what is not goes
  * through aphro_windowed_attention and aphro_differential_norm_gate. */

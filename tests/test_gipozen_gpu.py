@@ -390,11 +390,13 @@ def test_router_choice_uses_the_correction_and_the_weight_does_not(mops, outputs
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(72, 88, 5, 1, 2, True), (96, 64, 3, 0, 1, False), (75, 40, 4, 2, 3, True), (128, 32, 9, 1, 4, True)])
+@pytest.mark.parametrize("shape", [(72, 88, 5, 1, 2, True, 45), (96, 64, 3, 0, 1, False, 45), (75, 40, 4, 2, 3, True, 45),
+                                   (128, 32, 9, 1, 4, True, 45),
+                                   # steps in which an expert has dozens / hundreds of rows: blocks of 64 and of 128 rows
+                                   (128, 64, 3, 0, 2, False, 110), (128, 192, 3, 1, 2, True, 900), (192, 80, 2, 0, 2, False, 600)])
 def test_experts_against_the_restatement_and_alone(mops, dtype, shape):
-    width, ff, E, ident, top, shared = shape
+    width, ff, E, ident, top, shared, T = shape
     rng = np.random.default_rng(width + ff)
-    T = 45
     cfg = U.make_config([U.attention_layer(mlp="moe", ff=ff, experts=E, identity=ident, top=top, shared_ff=56 if shared else 0)], width=width)
     W = {k[7:]: rounded(v, dtype) for k, v in U.make_weights(cfg, seed=1).items() if k.startswith("l0.mlp.")}
     h = rounded(rng.standard_normal((T, width)), dtype)
@@ -414,11 +416,11 @@ def test_experts_against_the_restatement_and_alone(mops, dtype, shape):
         m.shared_down.weight.copy_(dev(W["shared.down"], dtype))
     with torch.no_grad():
         got = m(dev(h, dtype)).float().cpu().numpy()
-        one = torch.cat([m(dev(h[t:t + 1], dtype)) for t in (0, 17, 44)]).float().cpu().numpy()
+        one = torch.cat([m(dev(h[t:t + 1], dtype)) for t in (0, 17, T - 1)]).float().cpu().numpy()
     tol = 1e-4 if dtype == torch.float32 else 6e-2
     np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
     # a token's output does not depend on what else is in the batch
-    np.testing.assert_allclose(one, got[[0, 17, 44]], rtol=1e-6 if dtype == torch.float32 else 1e-2, atol=1e-6 if dtype == torch.float32 else 1e-2)
+    np.testing.assert_allclose(one, got[[0, 17, T - 1]], rtol=1e-6 if dtype == torch.float32 else 1e-2, atol=1e-6 if dtype == torch.float32 else 1e-2)
 
 
 # ---------------------------------------------------------------------------------------------------------------------
