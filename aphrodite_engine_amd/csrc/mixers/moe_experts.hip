@@ -154,7 +154,8 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(void* __restrict__ o
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+  constexpr int UNR = MT == 1 ? 8 : 2;                      // streaming weights: many pieces in flight per wave
+#pragma unroll UNR
   for (int k0 = 0; k0 < K; k0 += 32) {
     const u32x4 wf0 = *reinterpret_cast<const u32x4*>(w0 + k0);
     const u32x4 wf1 = *reinterpret_cast<const u32x4*>(w1 + k0);
@@ -188,8 +189,11 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(void* __restrict__ o
 // Prompt-sized steps, blocks of 128 rows: a workgroup owns the block's 128 rows x 128 weight rows (the gated product: 64 output
 // columns, their gate rows and their up rows; the down product: 128 columns) and walks K in steps of 64: both tiles go through
 // LDS (16-byte chunks XOR-swizzled by row so that the 16 rows of a fragment read hit different banks), the next step's pieces are
-// in flight in registers while the current step's 32 products per wave run.  Waves 2 x 2: 64 rows x 64 weight rows each.
+// in flight in registers while the current step's products run.  Waves 2 x 2: 64 rows x 64 weight rows each, as 2 x 2 tiles of
+// v_mfma_f32_32x32x16_bf16 (twice the multiply-adds per operand byte read from LDS of the 16 x 16 form, which measured 1.3 times
+// slower here: LDS reads, not the matrix cores, were the limit).
 constexpr int TG_BM = 128, TG_BN = 128, TG_BK = 64;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 template <bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(void* __restrict__ out, const uint16_t* __restrict__ a, int64_t a_stride,
@@ -200,13 +204,18 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(void* __restrict__ 
   __shared__ __attribute__((aligned(16))) uint16_t a_lds[TG_BM * TG_BK];
   __shared__ __attribute__((aligned(16))) uint16_t w_lds[TG_BN * TG_BK];
   __shared__ int32_t slot_lds[TG_BM];
-  const int b = blockIdx.x;
-  if (b >= num_blocks[0]) return;
-  const int e = block_expert[b];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-  const int wm = wave >> 1, wn = wave & 1;
+  // Workgroups go to the 8 XCDs round-robin by their linear index and each XCD has its own L2.  XCD x takes the column groups
+  // x, x + 8, ... of every block, block after block: the few weight tiles of its column groups stay in its L2 over all blocks
+  // of an expert, and a block's rows are fetched once per XCD by workgroups that run side by side.
   const int ncols = GLU ? TG_BN / 2 : TG_BN;               // output columns of the workgroup
-  const int n0 = blockIdx.y * ncols;
+  const int ny = (N + ncols - 1) / ncols, nyx = (ny + 7) / 8;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int b = seq / nyx, y = (seq % nyx) * 8 + xcd;
+  if (b >= num_blocks[0] || y >= ny) return;
+  const int e = block_expert[b];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int n0 = y * ncols;
   if (threadIdx.x < TG_BM) slot_lds[threadIdx.x] = sorted_slots[b * TG_BM + threadIdx.x];
   // this thread's pieces of the two tiles: 4 + 4 chunks of 16 bytes per K step
   const uint16_t* ap[4];
@@ -226,17 +235,20 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(void* __restrict__ 
       wp[i] = w + ((int64_t)e * N + min(n0 + row, N - 1)) * K + 8 * ch;
     }
   }
-  f32x4 acc[4][4];                                          // [row tile][weight tile]
+  f32x16 acc[2][2];                                         // [row tile of 32][weight tile of 32]
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
   u32x4 ra[4], rw[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     ra[i] = *reinterpret_cast<const u32x4*>(ap[i]);
     rw[i] = *reinterpret_cast<const u32x4*>(wp[i]);
   }
+  const int l31 = lane & 31, lh = lane >> 5;
   for (int k0 = 0; k0 < K; k0 += TG_BK) {
     __syncthreads();                                        // the previous step is consumed
 #pragma unroll
@@ -252,50 +264,54 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(void* __restrict__ 
         rw[i] = *reinterpret_cast<const u32x4*>(wp[i] + k0 + TG_BK);
       }
     }
+    // v_mfma_f32_32x32x16_bf16: a lane brings row (lane & 31), k = 8 (lane >> 5) .. + 7 of each operand
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      u32x4 af[4], wf[4];
+    for (int kk = 0; kk < TG_BK / 16; ++kk) {
+      u32x4 af[2], wf[2];
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const int row = 64 * wm + 16 * mt + c;
-        af[mt] = *reinterpret_cast<const u32x4*>(&a_lds[row * TG_BK + 8 * ((4 * ks + g) ^ (row & 7))]);
+      for (int mt = 0; mt < 2; ++mt) {
+        const int row = 64 * wm + 32 * mt + l31;
+        af[mt] = *reinterpret_cast<const u32x4*>(&a_lds[row * TG_BK + 8 * ((2 * kk + lh) ^ (row & 7))]);
       }
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        // the gated product: weight tiles {2 wn, 2 wn + 1} are gate rows, {4 + 2 wn, 5 + 2 wn} the up rows of the same columns
-        const int tile = GLU ? ((nt >> 1) * 4 + 2 * wn + (nt & 1)) : 4 * wn + nt;
-        const int row = 16 * tile + c;
-        wf[nt] = *reinterpret_cast<const u32x4*>(&w_lds[row * TG_BK + 8 * ((4 * ks + g) ^ (row & 7))]);
+      for (int nt = 0; nt < 2; ++nt) {
+        // the gated product: weight tile wn holds gate rows, tile 2 + wn the up rows of the same 32 columns
+        const int row = 32 * (GLU ? 2 * nt + wn : 2 * wn + nt) + l31;
+        wf[nt] = *reinterpret_cast<const u32x4*>(&w_lds[row * TG_BK + 8 * ((2 * kk + lh) ^ (row & 7))]);
       }
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[nt]), __builtin_bit_cast(bf16x8, af[mt]),
+        for (int nt = 0; nt < 2; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wf[nt]), __builtin_bit_cast(bf16x8, af[mt]),
                                                                 acc[mt][nt], 0, 0, 0);
     }
   }
-  // a lane holds, per (row tile, weight tile), 4 consecutive weight rows 4 g .. 4 g + 3 of block row 64 wm + 16 mt + c
+  // a lane holds, per (row tile, weight tile) and quad q, the 4 consecutive weight rows 8 q + 4 (lane >> 5) .. + 3 of block row
+  // 64 wm + 32 mt + (lane & 31)
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int row = 64 * wm + 16 * mt + c;
+  for (int mt = 0; mt < 2; ++mt) {
+    const int row = 64 * wm + 32 * mt + l31;
     const int slot = slot_lds[row];
-    if (GLU) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int col = n0 + 32 * wn + 16 * j + 4 * g;
+    for (int q = 0; q < 4; ++q) {
+      if (GLU) {
+        const int col = n0 + 32 * wn + 8 * q + 4 * lh;
         if (col >= N) continue;
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = slot >= 0 ? clamped_glu_f(acc[mt][j][r], acc[mt][2 + j][r], limit, alpha) : 0.f;
+        for (int r = 0; r < 4; ++r)
+          v[r] = slot >= 0 ? clamped_glu_f(acc[mt][0][4 * q + r], acc[mt][1][4 * q + r], limit, alpha) : 0.f;
         *reinterpret_cast<u32x2*>((uint16_t*)out + (int64_t)(b * TG_BM + row) * N + col) =
             u32x2{pack2_16<true>(v[0], v[1]), pack2_16<true>(v[2], v[3])};
-      }
-    } else if (slot >= 0) {
+      } else if (slot >= 0) {
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int col = n0 + 64 * wn + 16 * nt + 4 * g;
-        if (col < N) *reinterpret_cast<f32x4*>((float*)out + (int64_t)slot * N + col) = acc[mt][nt];
+        for (int nt = 0; nt < 2; ++nt) {
+          const int col = n0 + 64 * wn + 32 * nt + 8 * q + 4 * lh;
+          if (col < N)
+            *reinterpret_cast<f32x4*>((float*)out + (int64_t)slot * N + col) =
+                f32x4{acc[mt][nt][4 * q], acc[mt][nt][4 * q + 1], acc[mt][nt][4 * q + 2], acc[mt][nt][4 * q + 3]};
+        }
       }
     }
   }
@@ -425,7 +441,8 @@ static int moe_gemm(bool glu, void* out, const void* a, int64_t a_stride, const 
   const bool mfma = dtype == APHRO_BF16 && N % 16 == 0 && K % 32 == 0 && a_stride % 8 == 0 && ((uintptr_t)a & 15) == 0 &&
                     ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0;
   if (mfma && bm == TG_BM && K % TG_BK == 0 && N % 4 == 0) {
-    const dim3 grid((unsigned)(capacity / bm), (unsigned)((N + (glu ? 63 : 127)) / (glu ? 64 : 128)));
+    const int64_t ny = (N + (glu ? 63 : 127)) / (glu ? 64 : 128);
+    const dim3 grid((unsigned)(8 * (capacity / bm) * ((ny + 7) / 8)));
     if (glu)
       hipLaunchKernelGGL((moe_gemm_tiled_kernel<true>), grid, dim3(256), 0, (hipStream_t)stream, out, (const uint16_t*)a, a_stride,
                          (const uint16_t*)w, sorted_slots, block_expert, num_blocks, top, N, K, limit, alpha);
