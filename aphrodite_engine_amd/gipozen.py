@@ -209,14 +209,22 @@ class GipozenForCausalLM(nn.Module):
         """Checkpoint names: embed, head, final.norm, l<i>.norm{1,2}, l<i>.dwa, l<i>.mix.{q,k,v}[.conv], l<i>.mix.{g,o,lq1,lk1,
         lq2,lk2}, l<i>.mlp.{up,down,act} or l<i>.mlp.{router,correction,e<j>.{gate,up,down},shared.{gate,up,down,sg}}."""
         expected, seen = set(self.expected_names()), set()
+        # a second norm's gain of a layer that has no feed-forward is never used: accepted and left aside
+        unused = {f"l{i}.norm2" for i, layer in enumerate(self.layers) if layer.mlp is None}
         for name, t in weights:
+            if name in unused:
+                continue
             if name not in expected:
                 raise ValueError(f"unexpected tensor {name!r} in a Gipozen checkpoint")
             seen.add(name)
             self._load_one(name, t)
-        missing = sorted(expected - seen)
+        missing = expected - seen
+        if "head" in missing:                    # no output matrix of its own: the embedding's
+            self.head = self.embed
+            missing.discard("head")
+        missing -= {n for n in missing if n.endswith(".mlp.correction")}      # no correction: the scores alone choose
         if missing:
-            raise ValueError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:4]}")
+            raise ValueError(f"checkpoint lacks {len(missing)} tensors, e.g. {sorted(missing)[:4]}")
 
     @staticmethod
     def _put(dst: torch.Tensor, t: torch.Tensor, name: str) -> None:

@@ -80,6 +80,18 @@ def test_checkpoint_fills_fused_projections_experts_and_caches(tmp_path):
             load_model(str(tmp_path / change), dtype=torch.float32, device="cpu")
 
 
+def test_checkpoint_without_output_matrix_or_with_an_unused_gain(tmp_path):
+    from aphrodite_engine_amd.loader import load_model
+    cfg = U.make_config([A(mlp=None), A(kv_from=0, mlp="moe")])
+    W = U.make_weights(cfg, seed=4)
+    del W["head"]
+    del W["l1.mlp.correction"]
+    W["l0.norm2"] = np.array(1.25, np.float32)
+    U.write_checkpoint(str(tmp_path), cfg, W)
+    m = load_model(str(tmp_path), dtype=torch.float32, device="cpu")
+    assert m.head is m.embed and float(m.layers[1].mlp.correction.abs().sum()) == 0.0
+
+
 def test_restatement_mask_convolution_and_average():
     assert [j for j in range(10) if O.visible(9, j, 3, 2)] == [0, 1, 7, 8, 9]
     assert [j for j in range(10) if O.visible(9, j, 3, 0)] == [7, 8, 9]
