@@ -3,7 +3,7 @@
 plus each mixer kernel alone against its roofline and against the like kernel of the Llama path.  Prints ONE JSON line;
 the default workload of bench.py is untouched by it.  The Gipozen stack: windowed differential attention (two maps of half the
 head size over shared values, window 1024 + 4 kept tokens, 4-tap convolutions), every second layer reading the previous
-layer's keys and values and carrying 16 + 2 experts (top 4, a quarter of the dense feed-forward each, one shared expert)
+layer's keys and values and carrying 16 + 1 experts (top 4, a quarter of the dense feed-forward each, one shared expert)
 instead of the PolyNorm feed-forward; its expert products are priced against the MFMA figure over the ACTIVE experts' flops.
 
 Rooflines used: 8 TB/s HBM for the memory-bound kernels (norms, activations, decode attention, the decode step of the
@@ -43,11 +43,11 @@ def fatudra_config(s):
 
 def gipozen_config(s):
     d = s["dim"] // 2                       # two maps of half the head size: q is as wide as a plain head's
-    mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": s["dim"], "conv": 4, "diff": 0.3,
+    mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": s["dim"], "conv": 4, "diff": 0.25,
              "mask": {"size": GIP_WINDOW, "keep_first": GIP_KEEP}, "scale": d ** -0.5}
     eff = s["ff"] // 4 // 32 * 32
     dense = {"kind": "dense", "ff": s["ff"]}
-    moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0}, "router": {"experts": GIP_EXPERTS, "identity": 2, "top": GIP_TOP},
+    moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0}, "router": {"experts": GIP_EXPERTS, "identity": 1, "top": GIP_TOP},
            "shared": {"ff": eff, "limit": 7.0}}
     layers = []
     for i in range(LAYERS):
@@ -289,7 +289,7 @@ def gipozen_kernel_section(s, prompt_len, batch, ctx, device):
             like={"kernel": "silu_and_mul", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * ff * 6 / lsec / HBM, 3)})
         # ---- experts: route, sort, both products, combine -- against the dense feed-forward's library products of equal active size
         h = torch.randn(T, W, device=device, dtype=bf)
-        R = GIP_EXPERTS + 2
+        R = GIP_EXPERTS + 1
         zr = torch.randn(T, R, device=device)
         ids, wts = mops.experts_route(zr, None, GIP_TOP)
         wgu = torch.randn(GIP_EXPERTS, 2 * eff, W, device=device, dtype=bf) * W ** -0.5

@@ -270,7 +270,7 @@ def test_fused_differential_attention_in_mixed_batches(mops, shape):
     assert mops.differential_window_attention_supported(H, G, d, e, torch.bfloat16)
     rng = np.random.default_rng(H * d + e)
     lens, block = (210, 77), 16
-    lam, diff, eps = 0.45, 0.3, 1e-5
+    lam, diff, eps = 0.45, 0.35, 1e-5
     seqs = []
     for T in lens:
         q = U.bf16_round(rng.standard_normal((T, H * 2 * d)))
