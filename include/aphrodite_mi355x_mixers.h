@@ -3,8 +3,10 @@
  *
  * MI355X (gfx950 / CDNA4) kernels of the sequence mixers that are not plain rotary softmax attention: layer norm around
  * an fp32 residual stream, gated activations, softmax attention over a paged cache with a tabulated distance bias and a
- * position-dependent query temperature, and gated outer-product memories (decay linear attention, mLSTM) with their state
- * in per-request slots.  Same conventions as aphrodite_mi355x.h: device pointers, sizes and a hipStream_t (void*); every
+ * position-dependent query temperature, gated outer-product memories (decay linear attention, mLSTM) with their state
+ * in per-request slots, and -- further down -- an fp32 residual stream averaged over depth with scalar-gain RMS norms, a
+ * polynomial-norm activation, short causal convolutions with per-request state, (differential) attention under a sliding
+ * window that keeps the first tokens, and routed experts on unquantised weights.  Same conventions as aphrodite_mi355x.h: device pointers, sizes and a hipStream_t (void*); every
  * entry point is asynchronous on `stream`, allocates nothing, never synchronises and returns APHRO_OK or a negative code;
  * aphro_mixers_last_error() describes the failure (thread-local).
  *
